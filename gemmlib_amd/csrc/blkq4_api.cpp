@@ -1,0 +1,303 @@
+// Host side of the C ABI: argument validation, error strings, kernel selection.  Plain C++ with no
+// HIP headers; device work is reached through the C functions declared in blkq4_device.h.
+//
+// Behaviour mirrors the reference dispatcher (reference: src/blkq4_f16_gemm_sm80.cu:38-531): same
+// checks in the same order, same return codes, same message texts.
+
+#include "ms_blkq4gemm.h"
+
+#include <cstdint>
+#include <string>
+
+#include "blkq4_device.h"
+
+#define BLKQ4_EXPORT __attribute__((visibility("default")))
+
+namespace {
+
+inline void set_error(std::string* err, std::string&& text) {
+  if (err) *err = std::move(text);
+}
+
+inline bool supported_block_size(int bs) { return bs == 16 || bs == 32 || bs == 64; }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr const char* kRowWiseMessage =
+    "Row-wise blocking (column_wise_blocking = false) is not implemented by this library";
+
+// reference: src/blkq4_f16_gemm_sm80.cu:155-203 (blkq4_quant_size_sm80_T)
+int quant_size(int block_size, bool column_wise, int rows, int columns, int64_t& w_size,
+               int64_t& meta_size, std::string* err) {
+  if (rows == 0 || columns == 0) {
+    set_error(err, "Empty problem size: " + std::to_string(rows) + "x" + std::to_string(columns));
+    return -1;
+  }
+  const int krow = column_wise ? block_size : 1;
+  const int kcol = column_wise ? 1 : block_size;
+  const int meta_rows = rows / krow;
+  const int meta_cols = columns / kcol;
+  // The reference divides by the meta extent (which is zero when the matrix is smaller than one
+  // block, a division by zero there); such shapes are reported as not quantizable here.
+  if (rows < 0 || (rows % 64) != 0 || meta_rows == 0 || (rows % meta_rows) != 0) {
+    set_error(err, "Cannot block quantize matrix with rows: " + std::to_string(rows));
+    return -1;
+  }
+  if (columns < 0 || (columns % 32) != 0 || meta_cols == 0 || (columns % meta_cols) != 0) {
+    set_error(err, "Cannot block quantize matrix with columns: " + std::to_string(columns));
+    return -1;
+  }
+  w_size = static_cast<int64_t>(rows / 2) * columns;
+  meta_size = static_cast<int64_t>(meta_rows) * meta_cols;
+  return 0;
+}
+
+int device_failure(int code, std::string* err) {
+  set_error(err, std::string("Kernel execution failed: ") + blkq4_dev_error_string(code));
+  return -1;
+}
+
+}  // namespace
+
+// reference: src/blkq4_f16_gemm_sm80.cu:431-463
+extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_size_sm80(int block_size, bool column_wise_blocking,
+                                                       int rows, int columns,
+                                                       int64_t& quant_weights_size,
+                                                       int64_t& quant_meta_size, void* err_msg_ptr) {
+  quant_weights_size = 0;
+  quant_meta_size = 0;
+  auto* err = static_cast<std::string*>(err_msg_ptr);
+  if (!supported_block_size(block_size)) {
+    set_error(err, "Unsupported block size: " + std::to_string(block_size));
+    return -1;
+  }
+  return quant_size(block_size, column_wise_blocking, rows, columns, quant_weights_size,
+                    quant_meta_size, err);
+}
+
+// reference: src/blkq4_f16_gemm_sm80.cu:465-531 and :205-314 (blkq4_quant_sm80_T)
+extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_sm80(int block_size, bool column_wise_blocking, int rows,
+                                                  int columns, int leadingDimension, void* stream,
+                                                  void const* weights, size_t weights_size,
+                                                  void* quant_weights, size_t quant_weights_size,
+                                                  void* quant_scales, size_t quant_scales_size,
+                                                  void* offsets, size_t offsets_size,
+                                                  void* err_msg_ptr) {
+  auto* err = static_cast<std::string*>(err_msg_ptr);
+  if (!supported_block_size(block_size)) {
+    set_error(err, "Unsupported block size: " + std::to_string(block_size));
+    return -1;
+  }
+  const bool has_offsets = offsets != nullptr && offsets_size > 0;
+
+  if (rows == 0 || columns == 0) {
+    set_error(err, "Empty problem size: " + std::to_string(rows) + "x" + std::to_string(columns));
+    return -1;
+  }
+  int64_t w_elems = 0, meta_elems = 0;
+  if (int e = quant_size(block_size, column_wise_blocking, rows, columns, w_elems, meta_elems, err)) {
+    return e;
+  }
+  // element counts of the caller's buffers, as the reference's spans see them
+  const int64_t qw_have = static_cast<int64_t>(quant_weights_size);
+  const int64_t sc_have = static_cast<int64_t>(quant_scales_size / 2);
+  const int64_t zp_have = static_cast<int64_t>(offsets_size);
+  const int64_t w_have = static_cast<int64_t>(weights_size / 2);
+  if (qw_have < w_elems) {
+    set_error(err, "Unexpected quantized weight tensor size: " + std::to_string(qw_have) +
+                       " expected: " + std::to_string(w_elems));
+    return -1;
+  }
+  if (sc_have < meta_elems) {
+    set_error(err, "Unexpected scale tensor size: " + std::to_string(sc_have) +
+                       " expected: " + std::to_string(meta_elems));
+    return -1;
+  }
+  if (has_offsets && zp_have < meta_elems) {
+    set_error(err, "Unexpected offset tensor size: " + std::to_string(zp_have) +
+                       " expected: " + std::to_string(meta_elems));
+    return -1;
+  }
+  const int64_t w_need = static_cast<int64_t>(columns) * leadingDimension;
+  if (w_have < w_need) {
+    set_error(err, "Unexpected weight tensor size: " + std::to_string(w_have) +
+                       " expected: " + std::to_string(w_need));
+    return -1;
+  }
+  if (leadingDimension < rows) {
+    set_error(err, "Leading dimension " + std::to_string(leadingDimension) +
+                       " is smaller than the number of rows: " + std::to_string(rows));
+    return -1;
+  }
+  if (!column_wise_blocking) {
+    set_error(err, kRowWiseMessage);
+    return -1;
+  }
+  if (weights == nullptr || quant_weights == nullptr || quant_scales == nullptr) {
+    set_error(err, "Null tensor pointer");
+    return -1;
+  }
+
+  blkq4_prepack_args args{};
+  args.block_size = block_size;
+  args.rows = rows;
+  args.columns = columns;
+  args.ld = leadingDimension;
+  args.src = weights;
+  args.packed_w = quant_weights;
+  args.scales = quant_scales;
+  args.zero_points = has_offsets ? offsets : nullptr;
+  args.stream = stream;
+  if (int code = blkq4_dev_prepack(&args)) return device_failure(code, err);
+  return 0;
+}
+
+// reference: src/blkq4_f16_gemm_sm80.cu:319-429 and :38-153 (blkq4_gemm_sm80_T)
+extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wise_blocking, int m,
+                                                 int n, int k, void* stream, void const* act_ptr,
+                                                 size_t a_size, void const* weights_ptr,
+                                                 size_t weights_size, void const* scales_ptr,
+                                                 size_t scales_size, void const* offsets_ptr,
+                                                 size_t offsets_size, void* output_ptr,
+                                                 size_t output_size, void* err_msg_ptr) {
+  auto* err = static_cast<std::string*>(err_msg_ptr);
+  if (!supported_block_size(block_size)) {
+    set_error(err, "Unsupported block size: " + std::to_string(block_size));
+    return -1;
+  }
+  const bool has_offsets = offsets_ptr != nullptr && offsets_size > 0;
+
+  if (m <= 0 || n <= 0 || k <= 0) {
+    set_error(err, "Empty problem size: " + std::to_string(m) + "x" + std::to_string(n) + "x" +
+                       std::to_string(k));
+    return -1;
+  }
+  const int krow = column_wise_blocking ? block_size : 1;
+  const int kcol = column_wise_blocking ? 1 : block_size;
+  const uint64_t M = static_cast<uint64_t>(m), N = static_cast<uint64_t>(n), K = static_cast<uint64_t>(k);
+
+  if (a_size != M * K * 2) {
+    set_error(err, "Unexpected activation tensor size: " + std::to_string(a_size) +
+                       " expected: " + std::to_string(M * K * 2));
+    return -1;
+  }
+  if (weights_size != (K / 2) * (N / 2) * 2) {
+    set_error(err, "Unexpected weight tensor size: " + std::to_string(weights_size) +
+                       " expected: " + std::to_string(K / 2 * N / 2 * 2));
+    return -1;
+  }
+  const uint64_t meta_elems = (K / krow) * (N / kcol);
+  if (scales_size != meta_elems * 2) {
+    set_error(err, "Unexpected scale tensor size: " + std::to_string(scales_size) +
+                       " expected: " + std::to_string(meta_elems * 2));
+    return -1;
+  }
+  if (output_size != M * N * 2) {
+    set_error(err, "Unexpected output tensor size: " + std::to_string(output_size) +
+                       " expected: " + std::to_string(M * N * 2));
+    return -1;
+  }
+  if (has_offsets && offsets_size != meta_elems) {
+    set_error(err, "Unexpected offsets tensor size: " + std::to_string(offsets_size) +
+                       " expected: " + std::to_string(meta_elems));
+    return -1;
+  }
+  // What the reference kernel's can_implement rejects
+  // (src/mickey/cutlass_ext/q4gemm/kernel/quantb_gemm.h:172-255).
+  if (!aligned16(act_ptr) || !aligned16(weights_ptr) || (k % 8) != 0) {
+    set_error(err, "Kernel execution failed: Error Misaligned Operand");
+    return -1;
+  }
+  // n % 32: the quantize entry point cannot produce buffers for any other n (columns % 32 rule).
+  if ((k % 64) != 0 || (k % krow) != 0 || (n % kcol) != 0 || (n % 32) != 0) {
+    set_error(err, "Kernel execution failed: Error Invalid Problem");
+    return -1;
+  }
+  if ((reinterpret_cast<uintptr_t>(scales_ptr) & 1u) != 0 || !aligned16(output_ptr) || (n % 8) != 0) {
+    set_error(err, "Kernel execution failed: Error Misaligned Operand");
+    return -1;
+  }
+  if (!column_wise_blocking) {
+    set_error(err, kRowWiseMessage);
+    return -1;
+  }
+  if (act_ptr == nullptr || weights_ptr == nullptr || scales_ptr == nullptr || output_ptr == nullptr) {
+    set_error(err, "Null tensor pointer");
+    return -1;
+  }
+
+  blkq4_gemm_args args{};
+  args.block_size = block_size;
+  args.m = m;
+  args.n = n;
+  args.k = k;
+  args.a = act_ptr;
+  args.packed_w = weights_ptr;
+  args.scales = scales_ptr;
+  args.zero_points = has_offsets ? offsets_ptr : nullptr;
+  args.c = output_ptr;
+  args.stream = stream;
+  // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
+  const int code = (m > 16) ? blkq4_dev_gemm(&args) : blkq4_dev_skinny(&args);
+  if (code) return device_failure(code, err);
+  return 0;
+}
+
+extern "C" BLKQ4_EXPORT int blkq4_fp16_repack_sm80(int to_sm80, int rows, int columns, void* stream,
+                                                   void const* src, size_t src_size, void* dst,
+                                                   size_t dst_size, void* err_msg_ptr) {
+  auto* err = static_cast<std::string*>(err_msg_ptr);
+  if (rows <= 0 || columns <= 0) {
+    set_error(err, "Empty problem size: " + std::to_string(rows) + "x" + std::to_string(columns));
+    return -1;
+  }
+  if ((rows % 64) != 0) {
+    set_error(err, "Cannot block quantize matrix with rows: " + std::to_string(rows));
+    return -1;
+  }
+  if ((columns % 32) != 0) {
+    set_error(err, "Cannot block quantize matrix with columns: " + std::to_string(columns));
+    return -1;
+  }
+  const uint64_t bytes = static_cast<uint64_t>(rows / 2) * static_cast<uint64_t>(columns);
+  if (src_size != bytes || dst_size != bytes) {
+    set_error(err, "Unexpected quantized weight tensor size: " +
+                       std::to_string(src_size != bytes ? src_size : dst_size) +
+                       " expected: " + std::to_string(bytes));
+    return -1;
+  }
+  if (src == nullptr || dst == nullptr) {
+    set_error(err, "Null tensor pointer");
+    return -1;
+  }
+  {
+    const auto s = reinterpret_cast<uintptr_t>(src), d = reinterpret_cast<uintptr_t>(dst);
+    if (s < d + bytes && d < s + bytes) {
+      set_error(err, "Source and destination buffers overlap");
+      return -1;
+    }
+    if ((s & 15u) != 0 || (d & 15u) != 0) {
+      set_error(err, "Kernel execution failed: Error Misaligned Operand");
+      return -1;
+    }
+  }
+  blkq4_repack_args args{};
+  args.to_sm80 = to_sm80 ? 1 : 0;
+  args.rows = rows;
+  args.columns = columns;
+  args.src = src;
+  args.dst = dst;
+  args.stream = stream;
+  if (int code = blkq4_dev_repack(&args)) return device_failure(code, err);
+  return 0;
+}
+
+extern "C" BLKQ4_EXPORT void* blkq4_error_message_create(void) { return new std::string(); }
+
+extern "C" BLKQ4_EXPORT char const* blkq4_error_message_cstr(void* error_message) {
+  return error_message ? static_cast<std::string*>(error_message)->c_str() : "";
+}
+
+extern "C" BLKQ4_EXPORT void blkq4_error_message_destroy(void* error_message) {
+  delete static_cast<std::string*>(error_message);
+}

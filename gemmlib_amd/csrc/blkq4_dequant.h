@@ -1,0 +1,72 @@
+// Device helpers shared by the GEMM kernels: vector types for the MFMA builtins and the
+// nibble -> fp16 conversion applied in registers right before an MFMA.
+//
+// Dequantized value: fp16( scale * (q - zp) ) with ONE rounding -- bit-identical to the reference's
+// host-side dequantization (reference: test/blkq4_fp16_gemm_sm80_test.cu:314-328).  The packed word
+// layout (see blkq4_device.h) puts the pair (k0+2i, k0+2i+1) at nibble positions i and i+4, so
+//   (w & 0x000f000f) | 0x64006400  is the fp16 pair (1024 + q, 1024 + q)   (ulp of 1024 is 1)
+//   (w & 0x00f000f0) | 0x54005400  is the fp16 pair (  64 + q,   64 + q)   (ulp of 64 is 1/16)
+// and one shift by 8 exposes the other two pairs the same way.  Adding -(1024 + zp) resp. -(64 + zp)
+// is exact (small integers), the multiplication by the scale rounds once.  Per 8 weights: 1 shift,
+// 4 and-or, 4 packed adds, 4 packed multiplies.
+
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace blkq4 {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ half2_t as_half2(uint32_t x) { return __builtin_bit_cast(half2_t, x); }
+__device__ __forceinline__ uint32_t as_u32(half2_t x) { return __builtin_bit_cast(uint32_t, x); }
+
+// Per-(block, column) constants of the conversion.
+struct DequantConsts {
+  half2_t scale2;  // (s, s)
+  half2_t neg_c0;  // (-(1024 + zp), -(1024 + zp))
+  half2_t neg_c1;  // (-(64 + zp),   -(64 + zp))
+};
+
+// scale_bits: fp16 bit pattern; zp: 0..15
+__device__ __forceinline__ DequantConsts make_dequant_consts(uint32_t scale_bits, uint32_t zp) {
+  DequantConsts c;
+  c.scale2 = as_half2(scale_bits | (scale_bits << 16));
+  const uint32_t c0 = 0xE400u | zp;         // -(1024 + zp): 0x6400 is 1024.0, ulp 1, sign bit set
+  const uint32_t c1 = 0xD400u | (zp << 4);  // -(64 + zp):   0x5400 is 64.0, ulp 1/16, sign bit set
+  c.neg_c0 = as_half2(c0 | (c0 << 16));
+  c.neg_c1 = as_half2(c1 | (c1 << 16));
+  return c;
+}
+
+// One packed word (8 weights k0..k0+7 of one column) -> 8 fp16 in k order.
+__device__ __forceinline__ half8_t dequant_word(uint32_t w, const DequantConsts& c) {
+  const uint32_t y = w >> 8;
+  const half2_t p0 = (as_half2((w & 0x000f000fu) | 0x64006400u) + c.neg_c0) * c.scale2;  // k0, k0+1
+  const half2_t p1 = (as_half2((w & 0x00f000f0u) | 0x54005400u) + c.neg_c1) * c.scale2;  // k0+2, k0+3
+  const half2_t p2 = (as_half2((y & 0x000f000fu) | 0x64006400u) + c.neg_c0) * c.scale2;  // k0+4, k0+5
+  const half2_t p3 = (as_half2((y & 0x00f000f0u) | 0x54005400u) + c.neg_c1) * c.scale2;  // k0+6, k0+7
+  half8_t r;
+  r[0] = p0[0]; r[1] = p0[1];
+  r[2] = p1[0]; r[3] = p1[1];
+  r[4] = p2[0]; r[5] = p2[1];
+  r[6] = p3[0]; r[7] = p3[1];
+  return r;
+}
+
+__device__ __forceinline__ half8_t as_half8(uint4 v) {
+  uint4_t t = {v.x, v.y, v.z, v.w};
+  return __builtin_bit_cast(half8_t, t);
+}
+
+__device__ __forceinline__ uint16_t float_to_half_bits(float f) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+
+}  // namespace blkq4

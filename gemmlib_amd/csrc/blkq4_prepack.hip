@@ -1,0 +1,296 @@
+// Fused quantize + pack kernel and the layout conversion kernels (gfx950).
+//
+// One pass: every fp16 weight is read once (coalesced 16-byte loads along K), the block range is
+// reduced across the 2/4/8 neighbouring lanes that share a quantization block, scale and zero-point
+// are derived, the eight weights a lane holds become one packed 32-bit word, and words, scales and
+// zero-points leave through LDS so that global stores are coalesced in the packed layouts described
+// in blkq4_device.h.  No temporary device buffers.
+//
+// Arithmetic (every rounding point) follows the reference quantizer
+// (reference: src/mickey/blk_q4/f16_quant_sm80.cuh:96-141 and :261-313):
+//   fp16 -> fp32 exactly; min/max with strict compares in ascending k; asymmetric: range widened to
+//   include 0, scale_f = (max - min) / 15 (IEEE divide), zp = roundf(0 - min / scale_f) clamped to
+//   0..15, scale = fp16(scale_f); symmetric: scale = fp16(extreme / -8) with ties going to min;
+//   q = clamp(roundf(fmaf(v, 1 / float(scale), zp)), 0, 15) with the fp16-rounded scale re-read.
+
+#include <hip/hip_runtime.h>
+
+#include <stdint.h>
+
+#include "blkq4_device.h"
+
+namespace {
+
+constexpr int kTileN = 64;    // columns (n) per workgroup
+constexpr int kTileK = 256;   // rows (k) per workgroup
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
+}
+
+__device__ __forceinline__ uint16_t float_to_half_bits(float f) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));  // v_cvt_f16_f32, round to nearest even
+}
+
+// nibble position of weight t (0..7) inside its 32-bit word
+__device__ __forceinline__ constexpr int nibble_shift(int t) { return 4 * ((t >> 1) + 4 * (t & 1)); }
+
+template <int BS, bool HAS_ZP, bool ALIGNED>
+__global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __restrict__ src, int K,
+                                                           int N, int ld,
+                                                           uint4* __restrict__ packed_w,
+                                                           uint16_t* __restrict__ scales,
+                                                           uint8_t* __restrict__ zps) {
+  constexpr int kLanesPerBlock = BS / 8;     // lanes sharing one quantization block
+  constexpr int kBlocksPerTile = kTileK / BS;  // quantization blocks along K in one tile
+  __shared__ uint32_t w_lds[kTileK / 32][kTileN][4];
+  __shared__ uint16_t s_lds[kBlocksPerTile][kTileN];
+  __shared__ uint8_t z_lds[kBlocksPerTile][kTileN];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int n0 = blockIdx.x * kTileN;
+  const int k0 = blockIdx.y * kTileK;
+
+  const int kl = (lane & 31) * 8;  // this lane's first k inside the tile
+  const bool k_ok = (k0 + kl) < K;  // K is a multiple of 64, so a lane's 8 weights are all in or all out
+
+  // Issue every load of the wave first: 8 x 16 bytes per lane in flight.
+  uint4 raw[8];
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int nl = wave * 16 + it * 2 + (lane >> 5);
+    const int n = n0 + nl;
+    raw[it] = make_uint4(0, 0, 0, 0);
+    if (k_ok && n < N) {
+      const uint16_t* p = src + static_cast<size_t>(n) * ld + (k0 + kl);
+      if constexpr (ALIGNED) {
+        raw[it] = *reinterpret_cast<const uint4*>(p);
+      } else {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = static_cast<uint32_t>(p[2 * i]) | (static_cast<uint32_t>(p[2 * i + 1]) << 16);
+        raw[it] = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int nl = wave * 16 + it * 2 + (lane >> 5);
+    const uint32_t words[4] = {raw[it].x, raw[it].y, raw[it].z, raw[it].w};
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = half_bits_to_float(words[i] & 0xffffu);
+      v[2 * i + 1] = half_bits_to_float(words[i] >> 16);
+    }
+    // range over this lane's 8 weights, ascending k, strict compares (first of equal values wins)
+    float mn = v[0], mx = v[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) {
+      if (v[i] < mn) mn = v[i];
+      if (v[i] > mx) mx = v[i];
+    }
+    // ... and across the lanes of the block; "lower" holds the smaller k, which must win ties
+#pragma unroll
+    for (int mask = 1; mask < kLanesPerBlock; mask <<= 1) {
+      const float omn = __shfl_xor(mn, mask);
+      const float omx = __shfl_xor(mx, mask);
+      const bool lower = (lane & mask) == 0;
+      const float lo_mn = lower ? mn : omn, hi_mn = lower ? omn : mn;
+      const float lo_mx = lower ? mx : omx, hi_mx = lower ? omx : mx;
+      mn = (hi_mn < lo_mn) ? hi_mn : lo_mn;
+      mx = (hi_mx > lo_mx) ? hi_mx : lo_mx;
+    }
+
+    uint16_t scale_bits;
+    uint32_t zp;
+    if constexpr (HAS_ZP) {
+      // reference: range2scalezp, f16_quant_sm80.cuh:96-122
+      const float rmn = fminf(mn, 0.0f);
+      const float rmx = fmaxf(mx, 0.0f);
+      const float scale_f = __fdiv_rn(__fsub_rn(rmx, rmn), 15.0f);
+      float zero_point_fp = rmn;
+      if (scale_f != 0.0f) zero_point_fp = __fsub_rn(0.0f, __fdiv_rn(rmn, scale_f));
+      if (zero_point_fp < 0.0f) {
+        zp = 0;
+      } else if (zero_point_fp > 15.0f) {
+        zp = 15;
+      } else {
+        zp = static_cast<uint32_t>(roundf(zero_point_fp));
+      }
+      scale_bits = float_to_half_bits(scale_f);
+    } else {
+      // reference: range2scale, f16_quant_sm80.cuh:124-135
+      const float m = fabsf(mx) > fabsf(mn) ? mx : mn;
+      scale_bits = float_to_half_bits(__fdiv_rn(m, -8.0f));
+      zp = 8;
+    }
+
+    // reference: f16_quant_sm80.cuh:291-297 (scale re-read after fp16 rounding; -0.0 counts as zero)
+    const float scale = half_bits_to_float(scale_bits);
+    const float reciprocal_scale = (scale != 0.0f) ? __fdiv_rn(1.0f, scale) : 0.0f;
+    const float zp_f = static_cast<float>(zp);
+    uint32_t word = 0;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      float r = roundf(__fmaf_rn(v[t], reciprocal_scale, zp_f));
+      r = fmaxf(0.0f, fminf(15.0f, r));
+      word |= static_cast<uint32_t>(r) << nibble_shift(t);
+    }
+
+    w_lds[kl >> 5][nl][(kl >> 3) & 3] = word;
+    if ((lane & (kLanesPerBlock - 1)) == 0) {
+      s_lds[kl / BS][nl] = scale_bits;
+      if constexpr (HAS_ZP) z_lds[kl / BS][nl] = static_cast<uint8_t>(zp);
+    }
+  }
+  __syncthreads();
+
+  // packed weights: one 16-byte unit per thread and pass, 1 KiB contiguous per wave
+#pragma unroll
+  for (int r = 0; r < (kTileK / 32) * kTileN / kThreads; ++r) {
+    const int u = tid + r * kThreads;
+    const int ksl = u / kTileN;
+    const int nl = u % kTileN;
+    const int k = k0 + ksl * 32;
+    const int n = n0 + nl;
+    if (k < K && n < N) {
+      const uint4 val = *reinterpret_cast<const uint4*>(&w_lds[ksl][nl][0]);
+      packed_w[static_cast<size_t>(k >> 5) * N + n] = val;
+    }
+  }
+  // scales / zero-points: row-major [K/BS][N]
+#pragma unroll
+  for (int r = 0; r < (kBlocksPerTile * kTileN + kThreads - 1) / kThreads; ++r) {
+    const int u = tid + r * kThreads;
+    const int bl = u / kTileN;
+    const int nl = u % kTileN;
+    const int k = k0 + bl * BS;
+    const int n = n0 + nl;
+    if (bl < kBlocksPerTile && k < K && n < N) {
+      const size_t idx = static_cast<size_t>(k / BS) * N + n;
+      scales[idx] = s_lds[bl][nl];
+      if constexpr (HAS_ZP) zps[idx] = z_lds[bl][nl];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Layout conversion between the packed layout above and the reference's sm80 layout
+// (reference: src/mickey/blk_q4/f16_quant_sm80.cuh:362-417): uint8[K, N/2] column-major, where for
+// each 16x16 weight tile at (k0, n0), row in 0..3, col in 0..7, s in 0..3 the byte at
+// (k0 + 4*row + s, n0/2 + col) holds  low = q(k0 + 2*row + (s>>1), n0 + col + 8*(s&1))  and
+// high = the same with k + 8.  One thread converts one 16-byte unit (32 k of one n).
+// ------------------------------------------------------------------------------------------------
+
+template <bool TO_SM80>
+__global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__ src,
+                                                     uint8_t* __restrict__ dst, int K, int N) {
+  const size_t unit = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t units = static_cast<size_t>(K / 32) * N;
+  if (unit >= units) return;
+  const int ks = static_cast<int>(unit / N);
+  const int n = static_cast<int>(unit % N);
+  const int hi_n = (n & 15) >> 3;
+  const size_t pc = static_cast<size_t>((n & ~15) >> 1) + (n & 7);
+  const size_t col_base = pc * K + static_cast<size_t>(ks) * 32;
+
+  if constexpr (TO_SM80) {
+    const uint4 u = reinterpret_cast<const uint4*>(src)[unit];
+    const uint32_t words[4] = {u.x, u.y, u.z, u.w};
+    uint32_t q[32];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) q[8 * j + t] = (words[j] >> nibble_shift(t)) & 0xfu;
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+      for (int row = 0; row < 4; ++row)
+#pragma unroll
+        for (int odd = 0; odd < 2; ++odd) {
+          const int kk = 16 * tile + 2 * row + odd;
+          dst[col_base + 16 * tile + 4 * row + 2 * odd + hi_n] = static_cast<uint8_t>(q[kk] | (q[kk + 8] << 4));
+        }
+  } else {
+    uint32_t q[32];
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+      for (int row = 0; row < 4; ++row)
+#pragma unroll
+        for (int odd = 0; odd < 2; ++odd) {
+          const int kk = 16 * tile + 2 * row + odd;
+          const uint32_t b = src[col_base + 16 * tile + 4 * row + 2 * odd + hi_n];
+          q[kk] = b & 0xfu;
+          q[kk + 8] = b >> 4;
+        }
+    uint32_t words[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) words[j] |= q[8 * j + t] << nibble_shift(t);
+    reinterpret_cast<uint4*>(dst)[unit] = make_uint4(words[0], words[1], words[2], words[3]);
+  }
+}
+
+template <int BS>
+int launch_prepack(const blkq4_prepack_args* a) {
+  const dim3 grid((a->columns + kTileN - 1) / kTileN, (a->rows + kTileK - 1) / kTileK);
+  const dim3 block(kThreads);
+  hipStream_t stream = static_cast<hipStream_t>(a->stream);
+  const auto* src = static_cast<const uint16_t*>(a->src);
+  auto* pw = static_cast<uint4*>(a->packed_w);
+  auto* sc = static_cast<uint16_t*>(a->scales);
+  auto* zp = static_cast<uint8_t*>(a->zero_points);
+  const bool aligned = (reinterpret_cast<uintptr_t>(a->src) & 15u) == 0 && (a->ld % 8) == 0;
+  const bool has_zp = zp != nullptr;
+  if (has_zp) {
+    if (aligned) {
+      hipLaunchKernelGGL((prepack_kernel<BS, true, true>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, pw, sc, zp);
+    } else {
+      hipLaunchKernelGGL((prepack_kernel<BS, true, false>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, pw, sc, zp);
+    }
+  } else {
+    if (aligned) {
+      hipLaunchKernelGGL((prepack_kernel<BS, false, true>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, pw, sc, zp);
+    } else {
+      hipLaunchKernelGGL((prepack_kernel<BS, false, false>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, pw, sc, zp);
+    }
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace
+
+extern "C" int blkq4_dev_prepack(const blkq4_prepack_args* a) {
+  if ((reinterpret_cast<uintptr_t>(a->packed_w) & 15u) != 0) return static_cast<int>(hipErrorInvalidValue);
+  switch (a->block_size) {
+    case 16: return launch_prepack<16>(a);
+    case 32: return launch_prepack<32>(a);
+    case 64: return launch_prepack<64>(a);
+    default: return static_cast<int>(hipErrorInvalidValue);
+  }
+}
+
+extern "C" int blkq4_dev_repack(const blkq4_repack_args* a) {
+  const size_t units = static_cast<size_t>(a->rows / 32) * a->columns;
+  const dim3 grid(static_cast<unsigned>((units + 255) / 256));
+  hipStream_t stream = static_cast<hipStream_t>(a->stream);
+  const auto* src = static_cast<const uint8_t*>(a->src);
+  auto* dst = static_cast<uint8_t*>(a->dst);
+  if (a->to_sm80) {
+    hipLaunchKernelGGL((repack_kernel<true>), grid, dim3(256), 0, stream, src, dst, a->rows, a->columns);
+  } else {
+    hipLaunchKernelGGL((repack_kernel<false>), grid, dim3(256), 0, stream, src, dst, a->rows, a->columns);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+extern "C" const char* blkq4_dev_error_string(int code) {
+  return hipGetErrorString(static_cast<hipError_t>(code));
+}

@@ -1,0 +1,116 @@
+/*
+ * Public C ABI of the MI355X (gfx950) blockwise-int4 x fp16 GEMM library.
+ *
+ * The first three entry points keep the names, argument order, argument meaning and error behaviour
+ * of the reference library's public header (reference: include/ms_blkq4gemm.h:41-50, :71-80, :94-100,
+ * implemented in src/blkq4_f16_gemm_sm80.cu:319-531) so that a program or extension linked against
+ * the reference links against this library unchanged.  The `_sm80` suffix is part of that contract
+ * and says nothing about the hardware the code runs on.
+ *
+ * Conventions shared by all entry points
+ *   - every pointer is DEVICE memory owned by the caller unless stated otherwise;
+ *   - every `*_size` argument is a size in BYTES; the two outputs of the size query are ELEMENT counts;
+ *   - `stream` is a hipStream_t cast to void* (nullptr = the default stream); calls are asynchronous
+ *     with respect to that stream and allocate no device memory;
+ *   - `error_message` is nullptr or a `std::string*` that receives a message when the call fails;
+ *   - the return value is 0 on success and -1 on failure; no exception crosses the boundary;
+ *   - the library keeps no global state and may be called from several host threads.
+ *
+ * The includer provides <cstdint> and <cstddef> (as with the reference header).
+ */
+
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+
+extern "C" {
+
+/**
+ * C[m,n] (fp16, row-major) = A[m,k] (fp16, row-major) x dequant(W[k,n]), fp32 accumulation, one
+ * rounding to fp16.  W, scales and offsets are the buffers `blkq4_fp16_quant_sm80` produced for the
+ * same block_size / blocking / shape (or buffers converted with `blkq4_fp16_repack_sm80`).
+ *
+ * Replaces: reference include/ms_blkq4gemm.h:41-50 (src/blkq4_f16_gemm_sm80.cu:319-429).
+ *
+ * Sizes must be exact: a_size = m*k*2, weights_size = k*n/2, scales_size = (k/bs)*n*2,
+ * offsets_size = (k/bs)*n (or offsets_ptr == nullptr / offsets_size == 0 for symmetric weights with
+ * the implicit zero-point 8), output_size = m*n*2.  k must be a multiple of 64 and n a multiple of
+ * the block's column extent; A, W and C must be 16-byte aligned.
+ */
+int blkq4_fp16_gemm_sm80(
+  int block_size,
+  bool column_wise_blocking,
+  int m, int n, int k, void* stream,
+  void const* act_ptr, size_t a_size,
+  void const* weights_ptr, size_t weights_size,
+  void const* scales_ptr, size_t scales_size,
+  void const* offsets_ptr, size_t offsets_size,
+  void* output_ptr, size_t output_size,
+  void* error_message);
+
+/**
+ * Quantize an fp16 weight matrix blockwise to 4 bits and pack it for the GEMM above.
+ * `weights` holds element (row r, column c) at weights[r + c * leadingDimension] (rows = in_features,
+ * columns = out_features, i.e. a torch [out, in] contiguous tensor with leadingDimension = in).
+ *
+ * Replaces: reference include/ms_blkq4gemm.h:71-80 (src/blkq4_f16_gemm_sm80.cu:465-531).
+ *
+ * Outputs: quant_weights rows*columns/2 bytes; quant_scales one fp16 per block; offsets one uint8
+ * (0..15) per block, or nullptr / size 0 to select the symmetric quantizer.  The scale and offset
+ * buffers are byte-identical to the reference's for column-wise blocking (row-major [rows/bs, columns]).
+ * The weight buffer holds the same nibbles in this library's gfx950 order; `blkq4_fp16_repack_sm80`
+ * converts either way without loss.
+ */
+extern int blkq4_fp16_quant_sm80(
+    int block_size,
+    bool column_wise_blocking,
+    int rows, int columns, int leadingDimension,
+    void* stream,
+    void const* weights, size_t weights_size,
+    void* quant_weights, size_t quant_weights_size,
+    void* quant_scales, size_t quant_scales_size,
+    void* offsets, size_t offsets_size,
+    void* error_message);
+
+/**
+ * Element counts of the buffers `blkq4_fp16_quant_sm80` fills: quant_weights_size uint8 elements and
+ * quant_meta_size scale elements (and as many offset bytes).  Host-only.
+ *
+ * Replaces: reference include/ms_blkq4gemm.h:94-100 (src/blkq4_f16_gemm_sm80.cu:431-463).
+ */
+int blkq4_fp16_quant_size_sm80(
+    int block_size,
+    bool column_wise_blocking,
+    int rows, int columns,
+    int64_t& quant_weights_size,
+    int64_t& quant_meta_size,
+    void* error_message);
+
+/**
+ * Convert a packed weight buffer between this library's gfx950 order and the reference's sm80 order
+ * (reference: src/mickey/blk_q4/f16_quant_sm80.cuh:362-417).  `to_sm80 != 0` converts gfx950 -> sm80,
+ * `to_sm80 == 0` converts sm80 -> gfx950.  Both buffers hold rows*columns/2 bytes and must not
+ * overlap.  Scales and offsets need no conversion for column-wise blocking.
+ *
+ * No counterpart in the reference: it exists so that weights packed by the reference can be loaded
+ * here and vice versa, and so that the packing can be compared byte for byte with the reference's.
+ */
+int blkq4_fp16_repack_sm80(
+    int to_sm80,
+    int rows, int columns,
+    void* stream,
+    void const* src, size_t src_size,
+    void* dst, size_t dst_size,
+    void* error_message);
+
+/**
+ * Helpers for callers that cannot construct a C++ std::string (ctypes, cgo, JNI ...): create an
+ * error-message object to pass as `error_message`, read it, destroy it.  Host-only; no counterpart
+ * in the reference, whose callers are all C++.
+ */
+void* blkq4_error_message_create(void);
+char const* blkq4_error_message_cstr(void* error_message);
+void blkq4_error_message_destroy(void* error_message);
+
+}  // extern "C"
