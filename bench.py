@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the blkq4 hot path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs C4,C2,...] [--no-cpu]
+
+One "step" is one call of ``blkq4_fp16_gemm_sm80`` on the headline workload (C4: the M=2048 prefill
+GEMM); the GEMV (C2) and the other configurations are measured the same way and reported inside the
+same JSON line.  Inputs are resident in HBM before the timed region.  HBM-bound configurations rotate
+over enough distinct weight sets to exceed the 256 MB Infinity Cache.  Kernel time comes from HIP
+events on the launch stream around a captured graph of back-to-back launches; wall time around the
+same region gives ``value``.  The CPU baseline is the oracle (dequantize + fp32-accumulate GEMM,
+OpenMP) on a bounded sample of the same workload, and is only a baseline.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "blkq4 GEMM TFLOP/s (M=2048) + GEMV HBM GB/s (M=1), as % of MI355X roofline"
+PEAK_MFMA_TFLOPS = 2500.0   # fp16 dense MFMA, MI355X published
+PEAK_HBM_GBPS = 8000.0      # HBM3E, MI355X published
+INFINITY_CACHE_BYTES = 256 << 20
+
+# name: (M, K, N, block_size, has_offsets, bound)
+CONFIGS = {
+    "C1": (64, 1024, 1024, 32, True, "mfma"),
+    "C2": (1, 4096, 4096, 64, False, "hbm"),
+    "C3": (16, 4096, 11008, 32, True, "hbm"),
+    "C4": (2048, 4096, 4096, 64, True, "mfma"),
+    "C5": (4096, 8192, 28672, 16, True, "mfma"),
+}
+DESCRIPTION = {
+    "C1": "C1 CPU-runnable case M=64 K=1024 N=1024 bs32 asym",
+    "C2": "C2 decode GEMV M=1 K=4096 N=4096 bs64 sym",
+    "C3": "C3 skinny GEMM M=16 K=4096 N=11008 bs32 asym",
+    "C4": "C4 prefill GEMM M=2048 K=4096 N=4096 bs64 asym",
+    "C5": "C5 large-layer GEMM M=4096 K=8192 N=28672 bs16 asym",
+}
+
+
+def algorithmic(m, k, n, bs, has_offsets):
+    """FLOPs and bytes of one GEMM call: A + packed W + scales + zero-points (uint8) + C."""
+    flops = 2 * m * n * k
+    nbytes = 2 * m * k + k * n // 2 + 2 * k * n // bs + (k * n // bs if has_offsets else 0) + 2 * m * n
+    return flops, nbytes
+
+
+def prepack_bytes(k, n, bs, has_offsets):
+    return 2 * k * n + k * n // 2 + 2 * k * n // bs + (k * n // bs if has_offsets else 0)
+
+
+def timed_region(torch, launches, steps, warmup):
+    """launches: list of zero-argument callables that each enqueue ONE kernel on the current stream;
+    call i uses launches[i % len].  Returns (wall seconds, event seconds, 'graph'|'eager')."""
+    nl = len(launches)
+    for i in range(warmup):
+        launches[i % nl]()
+    torch.cuda.synchronize()
+    mode = "graph"
+    graph = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(steps):
+                    launches[i % nl]()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph.replay()  # untimed: first replay uploads the graph
+        torch.cuda.synchronize()
+    except Exception as e:  # pragma: no cover - depends on the runtime
+        sys.stderr.write(f"[bench] graph capture unavailable ({type(e).__name__}: {e}); timing eager launches\n")
+        graph = None
+        mode = "eager"
+        torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record()
+    if graph is not None:
+        graph.replay()
+    else:
+        for i in range(steps):
+            launches[i % nl]()
+    ev1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return t1 - t0, ev0.elapsed_time(ev1) * 1e-3, mode
+
+
+def make_problem(torch, capi, name, device, copies):
+    m, k, n, bs, has_offsets, _ = CONFIGS[name]
+    g = torch.Generator(device="cpu").manual_seed(1234 + list(CONFIGS).index(name))
+    a = torch.randn(m, k, generator=g, dtype=torch.float32).to(torch.float16).to(device)
+    w_elems, meta_elems = capi.quant_size(bs, True, k, n)
+    sets = []
+    w_host = None
+    for c in range(copies):
+        w_host = (torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).to(torch.float16)
+        w = w_host.to(device)
+        q_w = torch.empty(w_elems, dtype=torch.uint8, device=device)
+        q_s = torch.empty(meta_elems, dtype=torch.float16, device=device)
+        q_zp = torch.empty(meta_elems, dtype=torch.uint8, device=device) if has_offsets else None
+        capi.quant(bs, True, w, q_w, q_s, q_zp)
+        sets.append((q_w, q_s, q_zp))
+        del w
+    torch.cuda.synchronize()
+    out = torch.empty(m, n, dtype=torch.float16, device=device)
+    return a, sets, out, w_host
+
+
+def bench_gemm(torch, capi, name, device, steps, warmup):
+    m, k, n, bs, has_offsets, bound = CONFIGS[name]
+    flops, nbytes = algorithmic(m, k, n, bs, has_offsets)
+    copies = 1
+    if bound == "hbm":
+        per_set = nbytes - 2 * m * k - 2 * m * n
+        copies = INFINITY_CACHE_BYTES // per_set + 2
+    a, sets, out, w_host = make_problem(torch, capi, name, device, copies)
+
+    def mk(s):
+        q_w, q_s, q_zp = s
+        return lambda: capi.gemm(bs, True, m, n, k, a, q_w, q_s, q_zp, out)
+
+    launches = [mk(s) for s in sets]
+    wall, evt, mode = timed_region(torch, launches, steps, warmup)
+    per_call_wall = wall / steps
+    per_call_evt = evt / steps
+    if bound == "mfma":
+        achieved, peak, unit = flops / per_call_evt / 1e12, PEAK_MFMA_TFLOPS, "TFLOP/s"
+        value = flops / per_call_wall / 1e12
+    else:
+        achieved, peak, unit = nbytes / per_call_evt / 1e9, PEAK_HBM_GBPS, "GB/s"
+        value = nbytes / per_call_wall / 1e9
+    res = {
+        "workload": DESCRIPTION[name], "value": round(value, 3), "unit": unit,
+        "ms_per_step": round(per_call_wall * 1e3, 6), "kernel_us": round(per_call_evt * 1e6, 3),
+        "timing": mode, "weight_sets": copies, "flops": flops, "bytes": nbytes,
+        "tflops": round(flops / per_call_evt / 1e12, 3), "gbps": round(nbytes / per_call_evt / 1e9, 3),
+        "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+                     "frac": round(achieved / peak, 4), "traffic": None},
+    }
+    return res, (a, sets, out, w_host)
+
+
+def bench_prepack(torch, capi, device, steps, warmup):
+    _, k, n, bs, has_offsets, _ = CONFIGS["C5"]
+    nbytes = prepack_bytes(k, n, bs, has_offsets)
+    g = torch.Generator(device="cpu").manual_seed(4321)
+    w = (torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).to(torch.float16).to(device)
+    w_elems, meta_elems = capi.quant_size(bs, True, k, n)
+    q_w = torch.empty(w_elems, dtype=torch.uint8, device=device)
+    q_s = torch.empty(meta_elems, dtype=torch.float16, device=device)
+    q_zp = torch.empty(meta_elems, dtype=torch.uint8, device=device)
+    launches = [lambda: capi.quant(bs, True, w, q_w, q_s, q_zp)]
+    steps = max(10, steps // 10)
+    wall, evt, mode = timed_region(torch, launches, steps, max(2, warmup // 10))
+    per = evt / steps
+    ach = nbytes / per / 1e9
+    return {
+        "workload": "C5 quantize+prepack K=8192 N=28672 bs16 asym", "value": round(nbytes / (wall / steps) / 1e9, 3),
+        "unit": "GB/s", "ms_per_step": round(wall / steps * 1e3, 6), "kernel_us": round(per * 1e6, 3), "timing": mode,
+        "bytes": nbytes, "gbps": round(ach, 3),
+        "roofline": {"bound": "hbm", "achieved": round(ach, 3), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                     "frac": round(ach / PEAK_HBM_GBPS, 4), "traffic": None},
+    }
+
+
+def cpu_baseline(name, a_dev, w_host, target_seconds=12.0):
+    """The oracle's dequantize + GEMM on a bounded sample of rows of the same workload."""
+    import numpy as np
+    from oracle import blkq4_oracle as O
+    m, k, n, bs, has_offsets, _ = CONFIGS[name]
+    w = w_host.view(__import__("torch").int16).numpy().view(np.float16)
+    a = a_dev.cpu().view(__import__("torch").int16).numpy().view(np.float16)
+    t0 = time.perf_counter()
+    canon, s, z = O.quantize(bs, True, w, has_offsets)
+    t_quant = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    b = O.dequantize(bs, True, canon, s, z)
+    t_deq = time.perf_counter() - t0
+    rows = min(m, 16)
+    t0 = time.perf_counter()
+    O.gemm(np.ascontiguousarray(a[:rows]), b)
+    t_probe = time.perf_counter() - t0
+    rows = int(max(rows, min(m, rows * target_seconds / max(t_probe, 1e-3))))
+    t0 = time.perf_counter()
+    O.gemm(np.ascontiguousarray(a[:rows]), b)
+    t_gemm = time.perf_counter() - t0
+    flops = 2.0 * rows * n * k
+    return {
+        "value": round(flops / (t_gemm + t_deq * rows / m) / 1e12, 5), "unit": "TFLOP/s",
+        "cores": O.num_threads(), "kind": "port",
+        "sample": f"{rows} of {m} rows of {DESCRIPTION[name]}: dequantize {t_deq:.3f}s (whole B, charged pro rata), "
+                  f"GEMM {t_gemm:.3f}s; oracle quantize of B {t_quant:.3f}s "
+                  f"({prepack_bytes(k, n, bs, has_offsets) / t_quant / 1e9:.2f} GB/s)",
+    }
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args(argv)
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import torch
+    from gemmlib_amd import capi
+    capi.load()
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    wanted = [c.strip() for c in args.configs.split(",") if c.strip()]
+    results = {}
+    head = None
+    head_problem = None
+    for name in wanted:
+        if name == "prepack":
+            results["C5_prepack"] = bench_prepack(torch, capi, device, args.steps, args.warmup)
+        else:
+            res, problem = bench_gemm(torch, capi, name, device, args.steps, args.warmup)
+            results[name] = res
+            if name == "C4":
+                head, head_problem = res, problem
+            else:
+                del problem
+        torch.cuda.empty_cache()
+    if head is None:  # headline not requested: report the first one measured
+        head = next(iter(results.values()))
+
+    line = {
+        "metric": METRIC, "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": head["workload"], "timing": head.get("timing")},
+        "roofline": head["roofline"],
+    }
+    if "C2" in results:
+        line["gemv"] = {"workload": results["C2"]["workload"], "value": results["C2"]["value"], "unit": "GB/s",
+                        "kernel_us": results["C2"]["kernel_us"], "roofline": results["C2"]["roofline"]}
+    if not args.no_cpu and head_problem is not None:
+        a, sets, out, w_host = head_problem
+        line["cpu_baseline"] = cpu_baseline("C4", a, w_host)
+    line["all"] = results
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

@@ -127,6 +127,10 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
       // reference: range2scale, f16_quant_sm80.cuh:124-135
       const float m = fabsf(mx) > fabsf(mn) ? mx : mn;
       scale_bits = float_to_half_bits(__fdiv_rn(m, -8.0f));
+      // (+-0) / -8 is a zero of the opposite sign (an all-zero block gives the scale -0.0).  The
+      // compiler may evaluate the division as fma(m, -0.125, +0), which loses that sign, so the
+      // zero case takes its sign from the bits of m.
+      if (m == 0.0f) scale_bits = static_cast<uint16_t>((~__float_as_uint(m) >> 16) & 0x8000u);
       zp = 8;
     }
 

@@ -1,0 +1,165 @@
+"""GPU parity of the GEMM / GEMV path, through the C ABI, against the oracle's
+dequantize-then-GEMM (fp32 accumulation, one rounding to fp16).
+
+Two bars:
+  * the reference's own construction (test/blkq4_fp16_gemm_sm80_test.cu:194-256,469-472): weights from
+    the known-answer generator, activations on the 0.25 grid in [-4, 4]; every partial sum is exact in
+    fp32, so the output must be BIT-EXACT whatever the summation order;
+  * seeded Gaussian data (the benchmark configurations): max relative error <= 1e-2, where the error
+    of an output is measured against max(|ref|, 1e-3 * max|ref|).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import gemm_on_gpu, max_rel_err, quantize_on_gpu, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = 1e-2
+
+
+def grid_activations(rng, m, k):
+    """uniform on the 0.25 grid in [-4, 4] (cutlass TensorFillRandomUniform(view, seed, 4, -4, bits=2))."""
+    return (rng.integers(-16, 17, (m, k)) / 4.0).astype(np.float16)
+
+
+def run_kat(oracle, capi, device, bs, has_offsets, m, n, k):
+    rng = np.random.default_rng(m * 131 + n * 17 + k + bs + has_offsets)
+    kat = oracle.kat_generate(bs, True, k, n, has_offsets)
+    a = grid_activations(rng, m, k)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, kat["weights"], has_offsets)
+    # the quantizer must hand back the generator's data, otherwise the GEMM check below is moot
+    assert np.array_equal(to_np(q_w), oracle.native_from_canonical(kat["canon_w"]))
+    got = gemm_on_gpu(capi, device, bs, a, q_w, q_s, q_zp, n)
+    ref = oracle.gemm(a, kat["weights"])
+    if not np.array_equal(got.view(np.uint16), ref.view(np.uint16)):
+        bad = np.argwhere(got.view(np.uint16) != ref.view(np.uint16))
+        raise AssertionError(f"{bad.shape[0]} of {m * n} outputs differ, first {bad[:5].tolist()}: "
+                             f"got {got[tuple(bad[0])]} want {ref[tuple(bad[0])]}")
+
+
+# (block_size, has_offsets, m, n, k): the column-wise cases of the reference's test list
+# (test/blkq4_fp16_gemm_sm80_test.cu:501-518) ...
+REFERENCE_CASES = [
+    (16, False, 256, 672, 576), (16, True, 256, 672, 576),
+    (64, False, 256, 1024, 576), (64, True, 256, 1024, 576),
+    (16, False, 16, 672, 576), (16, True, 16, 672, 576),
+    (64, False, 16, 1024, 576), (64, True, 16, 1024, 576),
+]
+# ... the shapes it runs row-wise only, here column-wise (:480-493) ...
+EXTRA_CASES = [
+    (32, False, 32, 32, 64), (32, True, 32, 32, 64),
+    (32, False, 32, 96, 64), (32, True, 32, 96, 192),
+    (32, True, 256, 672, 576), (32, False, 512, 2048 + 32, 960),
+]
+# ... and what the reference never tests: M = 1, ragged M, M around the kernel switch at 16
+EDGE_CASES = [
+    (64, False, 1, 1024, 576), (32, True, 1, 96, 64), (16, True, 2, 160, 128), (32, True, 3, 672, 576),
+    (64, True, 7, 1024, 192), (16, False, 15, 704, 576), (32, True, 17, 96, 192), (64, True, 33, 288, 320),
+    (16, True, 65, 544, 256), (32, False, 100, 800, 448), (64, True, 129, 1056, 576), (32, True, 300, 256, 64),
+]
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES)
+def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
+    run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
+
+
+def gaussian_problem(seed, m, n, k):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    a = torch.randn(m, k, generator=g, dtype=torch.float32).to(torch.float16)
+    w = (torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).to(torch.float16)
+    return a.view(torch.int16).numpy().view(np.float16), w.view(torch.int16).numpy().view(np.float16)
+
+
+def run_gaussian(oracle, capi, device, bs, has_offsets, m, n, k, seed, sample_rows=None):
+    a, w = gaussian_problem(seed, m, n, k)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, w, has_offsets)
+    got = gemm_on_gpu(capi, device, bs, a, q_w, q_s, q_zp, n)
+    assert not np.isnan(got).any()
+    canon, s, z = oracle.quantize(bs, True, w, has_offsets)
+    b = oracle.dequantize(bs, True, canon, s, z)
+    rows = np.arange(m) if sample_rows is None else np.unique(
+        np.concatenate([[0, m - 1], np.random.default_rng(seed).integers(0, m, sample_rows)]))
+    ref = oracle.gemm(np.ascontiguousarray(a[rows]), b)
+    err = max_rel_err(got[rows], ref)
+    exact = float(np.mean(got[rows].view(np.uint16) == ref.view(np.uint16)))
+    print(f"m={m} n={n} k={k} bs={bs} zp={has_offsets}: max rel err {err:.3e}, bit-identical outputs {exact:.4f}")
+    assert err <= TOLERANCE
+    return got, q_w, q_s, q_zp, a
+
+
+def test_config1_cpu_runnable_case(oracle, capi, device):
+    run_gaussian(oracle, capi, device, 32, True, 64, 1024, 1024, seed=1235)
+
+
+def test_config2_decode_gemv(oracle, capi, device):
+    run_gaussian(oracle, capi, device, 64, False, 1, 4096, 4096, seed=1236)
+
+
+def test_config3_skinny(oracle, capi, device):
+    run_gaussian(oracle, capi, device, 32, True, 16, 11008, 4096, seed=1237)
+
+
+def test_config4_prefill(oracle, capi, device):
+    run_gaussian(oracle, capi, device, 64, True, 2048, 4096, 4096, seed=1238, sample_rows=96)
+
+
+def test_config5_large_layer(oracle, capi, device):
+    """full shape on the GPU; the oracle evaluates a sample of output rows, and linearity
+    (C(2a) = 2 C(a) exactly, scaling by 2 commutes with every rounding) covers the rest."""
+    m, n, k, bs = 4096, 28672, 8192, 16
+    got, q_w, q_s, q_zp, a = run_gaussian(oracle, capi, device, bs, True, m, n, k, seed=1239, sample_rows=6)
+    got2 = gemm_on_gpu(capi, device, bs, (a * np.float16(2)).astype(np.float16), q_w, q_s, q_zp, n)
+    # outputs in fp16's subnormal range gain one bit when doubled, so they are compared by distance
+    normal = np.abs(got) >= np.float16(2.0 ** -13)
+    twice = (got.astype(np.float32) * 2).astype(np.float16)
+    assert np.array_equal(twice[normal].view(np.uint16), got2[normal].view(np.uint16))
+    assert np.all(np.abs(twice[~normal].astype(np.float32) - got2[~normal].astype(np.float32)) <= 2.0 ** -23)
+
+
+@pytest.mark.parametrize("m", [1, 2, 4, 5, 8, 11, 16, 17, 31, 64, 96, 127, 128, 200])
+@pytest.mark.parametrize("bs,has_offsets", [(16, True), (32, False), (64, True)])
+def test_every_m_band(oracle, capi, device, m, bs, has_offsets):
+    run_gaussian(oracle, capi, device, bs, has_offsets, m, 352, 512, seed=m * 10 + bs)
+
+
+def test_rows_are_independent(oracle, capi, device):
+    """row r of C depends only on row r of A: the M=1 result equals row 0 of the M=16 and M=64 results."""
+    a, w = gaussian_problem(77, 64, 512, 1024)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, 32, w, True)
+    c64 = gemm_on_gpu(capi, device, 32, a, q_w, q_s, q_zp, 512)
+    c16 = gemm_on_gpu(capi, device, 32, a[:16], q_w, q_s, q_zp, 512)
+    c1 = gemm_on_gpu(capi, device, 32, a[:1], q_w, q_s, q_zp, 512)
+    assert max_rel_err(c16, c64[:16]) <= 2e-3   # different kernels, different summation order
+    assert max_rel_err(c1, c16[:1]) <= 2e-3
+
+
+def test_weights_repacked_from_reference_order(oracle, capi, device):
+    """a buffer in the reference's sm80 byte order (as the reference's quantizer would have written
+    it) converts with blkq4_fp16_repack_sm80 and gives the same GEMM result."""
+    rng = np.random.default_rng(8)
+    kat = oracle.kat_generate(32, True, 192, 96, True)
+    sm80_w, ps, pz = oracle.quant_sm80(32, True, kat["weights"], True)
+    src = to_dev(sm80_w, device)
+    dst = torch.empty_like(src)
+    capi.repack(False, 192, 96, src, dst)
+    a = grid_activations(rng, 32, 192)
+    got = gemm_on_gpu(capi, device, 32, a, dst, to_dev(ps, device), to_dev(pz, device), 96)
+    assert np.array_equal(got.view(np.uint16), oracle.gemm(a, kat["weights"]).view(np.uint16))
+
+
+def test_non_default_stream(oracle, capi, device):
+    a, w = gaussian_problem(5, 8, 256, 256)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, 64, w, True)
+    ref = gemm_on_gpu(capi, device, 64, a, q_w, q_s, q_zp, 256)
+    s = torch.cuda.Stream()
+    a_dev = to_dev(a, device)
+    out = torch.zeros((8, 256), dtype=torch.float16, device=device)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        capi.gemm(64, True, 8, 256, 256, a_dev, q_w, q_s, q_zp, out, stream=s)
+    s.synchronize()
+    assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16))

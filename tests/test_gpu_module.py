@@ -1,0 +1,72 @@
+"""The Python drop-in surface (ms_blkq4linear_ext + BlkQ4Linear) on the GPU, against the oracle.
+Mirrors what the reference's usage script does (reference: python/blkq4linear_test.py:10-85) and then
+goes further: it actually calls forward()."""
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import max_rel_err, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mod():
+    from gemmlib_amd import ms_blkq4linear  # fails loudly if the extension is not built
+    return ms_blkq4linear
+
+
+def test_quant_matches_known_answer(oracle, device, mod):
+    """the reference script's construction: in=64, out=32, block 32 (here column-wise)."""
+    from gemmlib_amd import ms_blkq4linear_ext as ext
+    kat = oracle.kat_generate(32, True, 64, 32, True)
+    q_w, q_s, q_zp = ext.quant(32, True, True, to_dev(kat["weights"], device))
+    assert q_w.dtype == torch.uint8 and q_w.dim() == 1 and q_w.numel() == 64 * 32 // 2
+    assert q_s.dtype == torch.float16 and q_s.numel() == 2 * 32 and q_zp.dtype == torch.uint8
+    assert np.array_equal(to_np(q_w), oracle.native_from_canonical(kat["canon_w"]))
+    assert np.array_equal(to_np(q_s).reshape(2, 32).view(np.uint16), kat["scales"].T.view(np.uint16))
+    assert np.array_equal(to_np(q_zp).reshape(2, 32), kat["zps"].T)
+
+
+@pytest.mark.parametrize("scale_only", [False, True])
+@pytest.mark.parametrize("m", [1, 16, 80])
+def test_module_forward_with_bias(oracle, device, mod, scale_only, m):
+    g = torch.Generator(device="cpu").manual_seed(3 + m)
+    k, n, bs = 512, 384, 64
+    w = (torch.randn(n, k, generator=g) * 0.02).to(torch.float16)
+    bias = torch.randn(n, generator=g).to(torch.float16)
+    x = torch.randn(m, k, generator=g).to(torch.float16)
+    layer = mod.BlkQ4Linear(bs, True, scale_only, w.to(device), bias.to(device))
+    assert layer.in_features == k and layer.out_features == n and layer.has_offsets == (not scale_only)
+    if scale_only:
+        assert layer.q_zp.numel() == 0 and layer.q_zp.device.type == "cuda"
+    y = layer(x.to(device))
+    assert y.shape == (m, n) and y.dtype == torch.float16
+    w_np = w.view(torch.int16).numpy().view(np.float16)
+    canon, s, z = oracle.quantize(bs, True, w_np, not scale_only)
+    ref = oracle.gemm(x.view(torch.int16).numpy().view(np.float16), oracle.dequantize(bs, True, canon, s, z))
+    ref = (torch.from_numpy(ref.view(np.int16)).view(torch.float16) + bias).view(torch.int16).numpy().view(np.float16)
+    assert max_rel_err(to_np(y), ref) <= 1e-2
+
+
+def test_extension_argument_checks(device, mod):
+    from gemmlib_amd import ms_blkq4linear_ext as ext
+    w = torch.zeros(32, 64, dtype=torch.float16, device=device)
+    with pytest.raises(RuntimeError, match="only supports float16 weights"):
+        ext.quant(32, True, True, w.float())
+    with pytest.raises(RuntimeError, match="only supports 2D tensors"):
+        ext.quant(32, True, True, w.reshape(2, 16, 64))
+    with pytest.raises(RuntimeError, match="only supports contiguous tensors"):
+        ext.quant(32, True, True, torch.zeros(64, 64, dtype=torch.float16, device=device)[:, ::2])
+    with pytest.raises(RuntimeError, match="only supports CUDA tensors"):
+        ext.quant(32, True, True, w.cpu())
+    with pytest.raises(RuntimeError, match="Unsupported block size: 48"):
+        ext.quant(48, True, True, w)
+    with pytest.raises(RuntimeError, match="Cannot block quantize matrix with rows: 96"):
+        ext.quant(32, True, True, torch.zeros(32, 96, dtype=torch.float16, device=device))
+    q_w, q_s, q_zp = ext.quant(32, True, True, w)
+    with pytest.raises(RuntimeError, match="Activation shape is not compatible"):
+        ext.forward(32, True, 64, 32, torch.zeros(4, 32, dtype=torch.float16, device=device), q_w, q_s, q_zp)
+    with pytest.raises(RuntimeError, match="only supports float16 inputs"):
+        ext.forward(32, True, 64, 32, torch.zeros(4, 64, device=device), q_w, q_s, q_zp)
