@@ -60,6 +60,34 @@ __device__ __forceinline__ half8_t dequant_word(uint32_t w, const DequantConsts&
   return r;
 }
 
+// The four literals of the conversion, held in VGPRs: with register operands `(w & mask) | magic`
+// is one v_and_or_b32 (a VOP3 instruction can carry at most one literal, so with literal operands
+// it becomes two instructions).  `opaque()` hides the value from constant propagation.
+struct DequantMasks {
+  uint32_t lo_mask, hi_mask, magic_1024, magic_64;
+  __device__ __forceinline__ static uint32_t opaque(uint32_t v) {
+    asm volatile("" : "+v"(v));
+    return v;
+  }
+  __device__ __forceinline__ static DequantMasks make() {
+    DequantMasks m;
+    m.lo_mask = opaque(0x000f000fu);
+    m.hi_mask = opaque(0x00f000f0u);
+    m.magic_1024 = opaque(0x64006400u);
+    m.magic_64 = opaque(0x54005400u);
+    return m;
+  }
+};
+
+// Pair `pair` (0..3) of a packed word: the fp16 values of weights k0 + 2*pair and k0 + 2*pair + 1.
+// `w_shifted` is the word itself for pairs 0/1 and the word shifted right by 8 for pairs 2/3.
+// Three instructions: v_and_or_b32, v_pk_add_f16, v_pk_mul_f16.
+__device__ __forceinline__ half2_t dequant_pair(uint32_t w_shifted, int pair, const DequantConsts& c,
+                                                const DequantMasks& m) {
+  if ((pair & 1) == 0) return (as_half2((w_shifted & m.lo_mask) | m.magic_1024) + c.neg_c0) * c.scale2;
+  return (as_half2((w_shifted & m.hi_mask) | m.magic_64) + c.neg_c1) * c.scale2;
+}
+
 __device__ __forceinline__ half8_t as_half8(uint4 v) {
   uint4_t t = {v.x, v.y, v.z, v.w};
   return __builtin_bit_cast(half8_t, t);
