@@ -47,9 +47,9 @@ namespace {
 
 using namespace blkq4;
 
-constexpr int kThreads = 256;
-constexpr int kWaves = 4;
-constexpr int kBN = 128;
+constexpr int kWaves = 8;  // two per SIMD
+constexpr int kThreads = 64 * kWaves;
+constexpr int kBN = 32 * kWaves;
 constexpr int kBK = 64;
 constexpr int kStages = 4;    // LDS ring depth
 constexpr int kDistance = 3;  // tiles requested ahead of the one being consumed
@@ -83,11 +83,12 @@ struct Stage {
   static constexpr int kBBytes = kWaves * 1024;              // [wave][lane] 16-byte units
   static constexpr int kMetaBytes = kWaves * kBlocks * 128;  // [wave][block][64 B scales | 32 B zps | pad]
   static constexpr int kBytes = kABytes + kBBytes + kMetaBytes;
-  static constexpr int kOps = RT + 1 + kBlocks;              // async copies per wave and stage
+  static constexpr int kAOps = (4 * RT + kWaves - 1) / kWaves;  // 8-row activation copies per wave and stage
+  static constexpr int kOps = kAOps + 1 + kBlocks;              // async copies per wave and stage
 };
 
 template <int BS, bool HAS_ZP, int RT>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mfma_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_mfma_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ S,
     const uint8_t* __restrict__ Z, uint16_t* __restrict__ C, int M, int N, int K, int m_tiles) {
   using St = Stage<BS, RT>;
@@ -114,10 +115,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   const int KT = K / kBK;
 
   // ---- per-lane byte offsets of the async copies inside k tile 0 ----
-  uint32_t a_off[RT];
+  constexpr int kAOps = St::kAOps;
+  uint32_t a_off[kAOps];
+  uint32_t a_dst[kAOps];  // LDS byte offset of the 8-row group inside the stage
 #pragma unroll
-  for (int p = 0; p < RT; ++p) {
-    const int row = 8 * (4 * p + wave) + (lane >> 3);  // row inside the tile
+  for (int p = 0; p < kAOps; ++p) {
+    // 4*RT groups of 8 rows are shared out over the waves; with fewer groups than waves the extra
+    // waves copy a group a second time (same bytes to the same place) so that every wave has the
+    // same number of copies in flight
+    const int group = (kWaves * p + wave) % (4 * RT);
+    a_dst[p] = group * 1024;
+    const int row = 8 * group + (lane >> 3);  // row inside the tile
     const int col = (lane & 7) ^ ((row >> 1) & 7);     // logical 16-byte column this lane fetches
     a_off[p] = static_cast<uint32_t>(min(m0 + row, M - 1)) * (static_cast<uint32_t>(K) * 2u) + col * 16;
   }
@@ -134,17 +142,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)(&lds[0])));  // LDS byte address
 
   // Async copy number q (0 .. kOps-1) of k tile `tile_` into ring slot `stage_`:
-  // q < RT: 8 activation rows; q == RT: this wave's packed weights; q > RT: one scale/zero-point row.
+  // q < kAOps: 8 activation rows; q == kAOps: this wave's packed weights; above: one scale/zero-point row.
 #define BLKQ4_COPY_OP(q_, tile_, stage_)                                                                  \
   {                                                                                                       \
     const uint32_t sbase_ = lds0 + (stage_) * St::kBytes;                                                 \
-    if ((q_) < RT) {                                                                                      \
-      async_copy_16(sbase_ + (4 * (q_) + wave) * 1024, A + static_cast<size_t>(tile_) * 128, a_off[(q_) < RT ? (q_) : 0]); \
-    } else if ((q_) == RT) {                                                                              \
+    if ((q_) < kAOps) {                                                                                   \
+      async_copy_16(sbase_ + a_dst[(q_) < kAOps ? (q_) : 0], A + static_cast<size_t>(tile_) * 128,       \
+                    a_off[(q_) < kAOps ? (q_) : 0]);                                                      \
+    } else if ((q_) == kAOps) {                                                                           \
       async_copy_16(sbase_ + St::kABytes + wave * 1024, W + static_cast<size_t>(tile_) * b_stride, b_off); \
     } else if (meta_active) {                                                                             \
-      async_copy_4_flat(sbase_ + St::kABytes + St::kBBytes + (wave * kBlocks + ((q_) - RT - 1)) * 128,    \
-                        meta_ptr + static_cast<size_t>((tile_) * kBlocks + ((q_) - RT - 1)) * meta_row_bytes); \
+      async_copy_4_flat(sbase_ + St::kABytes + St::kBBytes + (wave * kBlocks + ((q_) - kAOps - 1)) * 128,    \
+                        meta_ptr + static_cast<size_t>((tile_) * kBlocks + ((q_) - kAOps - 1)) * meta_row_bytes); \
     }                                                                                                     \
   }
 
@@ -337,11 +346,10 @@ int launch_one(const blkq4_gemm_args* a) {
 
 template <int BS, bool HAS_ZP>
 int launch_rt(const blkq4_gemm_args* a) {
-  // rows per workgroup: 256 unless the whole problem is shorter
+  // rows per workgroup: 128 unless the whole problem is shorter
   if (a->m <= 32) return launch_one<BS, HAS_ZP, 1>(a);
   if (a->m <= 64) return launch_one<BS, HAS_ZP, 2>(a);
-  if (a->m <= 128) return launch_one<BS, HAS_ZP, 4>(a);
-  return launch_one<BS, HAS_ZP, 8>(a);
+  return launch_one<BS, HAS_ZP, 4>(a);
 }
 
 template <int BS>
