@@ -3,7 +3,7 @@
 // The work is a stream over the packed weights (K*N/2 bytes plus scales and zero-points) that has to
 // run at HBM speed; everything else is arranged so that the stream is requested as early and as
 // deeply as possible and nothing serialises behind it:
-//   - a workgroup of four waves owns 16 (M <= 4) or 32 output columns and the whole K range; the waves split K in
+//   - a workgroup of four waves owns 16, 32 or 48 output columns and the whole K range; the waves split K in
 //     128-deep slices, so every wave load is one 16-byte unit per lane: 16 columns x 4 consecutive
 //     k-units = four contiguous 256-byte runs of the packed layout;
 //   - a wave keeps the weight units, scales and zero-points of kDepth slices in flight and refills a
@@ -42,8 +42,7 @@ struct Slot {
 };
 
 // DEPTH: k slices (128 deep) a wave keeps in flight.  NT: 16-column tiles per wave that share one
-// activation operand (NT = 2 for M > 4, where fetching the activation rows of a slice touches 16
-// different rows and costs more L1 tag look-ups than the weights themselves).
+// activation operand.
 template <int BS, bool HAS_ZP, int DEPTH, int NT>
 __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(const uint16_t* __restrict__ A,
                                                                const uint4* __restrict__ W,
@@ -59,7 +58,15 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(const uint16_t* _
   const int lane = tid & 63;
   const int nl = lane & 15;  // column inside the tile (weights operand) / activation row (other operand)
   const int g = lane >> 4;   // which of the 4 k-units of a slice
-  const int n = blockIdx.x * (16 * NT) + nl;  // column of tile 0; tile t is 16*t further
+  const int tiles = N >> 4;
+  // column this lane loads for tile t; a tile past the end (last workgroup only, when NT does not
+  // divide the tile count) re-reads the workgroup's first tile and is not stored
+  int n[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int tile = blockIdx.x * NT + t;
+    n[t] = ((tile < tiles) ? tile : blockIdx.x * NT) * 16 + nl;
+  }
   const bool row_ok = nl < M;
   const DequantMasks masks = DequantMasks::make();
   // lanes without a row load nothing and feed whatever their registers hold to the MFMA: an output
@@ -85,9 +92,9 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(const uint16_t* _
     const int ksg_ = ok_ ? ks_ : (ks_ & wrap_mask);                                            \
     const int b_ = (BS == 64) ? (ksg_ >> 1) : (BS == 32) ? ksg_ : (2 * ksg_);                  \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                           \
-      (dst_).w[t] = W[static_cast<size_t>(ksg_) * N + n + 16 * t];                             \
+      (dst_).w[t] = W[static_cast<size_t>(ksg_) * N + n[t]];                                  \
       _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                      \
-        const size_t mi_ = static_cast<size_t>(b_ + q) * N + n + 16 * t;                       \
+        const size_t mi_ = static_cast<size_t>(b_ + q) * N + n[t];                           \
         const uint32_t sc_ = S[mi_];                                                           \
         (dst_).sc[t][q] = ok_ ? sc_ : 0u;                                                      \
         (dst_).zp[t][q] = HAS_ZP ? static_cast<uint32_t>(Z[mi_]) : 8u;                         \
@@ -147,7 +154,7 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(const uint16_t* _
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) r[e] += red[((w * NT + t) * 64 + lane) * 4 + e];
       }
-      if (row_ok) {
+      if (row_ok && blockIdx.x * NT + t < tiles) {
         // lane (row nl, group g) holds output columns 4g .. 4g+3 of 16-column tile t
         const uint32_t lo = float_to_half_bits(r[0]) | (static_cast<uint32_t>(float_to_half_bits(r[1])) << 16);
         const uint32_t hi = float_to_half_bits(r[2]) | (static_cast<uint32_t>(float_to_half_bits(r[3])) << 16);
@@ -156,6 +163,30 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(const uint16_t* _
       }
     }
   }
+}
+
+// The kernel is bound by instruction issue as much as by the weight stream, so what matters is how
+// evenly the workgroups fill the 256 compute units: with T column tiles per workgroup the busiest
+// unit works through ceil(workgroups / 256) * T tiles.  Wider workgroups also re-read the activation
+// rows less often, which weighs more the more rows there are.
+void choose_shape(int m, int n, int* nt, int* depth) {
+  constexpr int kComputeUnits = 256;
+  const int tiles = n / 16;
+  const float a_weight = (m > 4) ? 0.2f : 0.05f;  // cost of fetching the activations relative to one tile's work
+  float best = 0.f;
+  *nt = 1;
+  for (int t = 1; t <= 3; ++t) {
+    const int wgs = (tiles + t - 1) / t;
+    const int rounds = (wgs + kComputeUnits - 1) / kComputeUnits;
+    const float cost = static_cast<float>(rounds) * (static_cast<float>(t) + a_weight);
+    if (t == 1 || cost < best) {
+      best = cost;
+      *nt = t;
+    }
+  }
+  // one tile per workgroup: 8 slices in flight while at most two workgroups share a unit, else 4
+  // (the deeper ring needs too many registers for more resident waves)
+  *depth = (*nt == 1 && tiles <= 2 * kComputeUnits) ? 8 : 4;
 }
 
 template <int BS>
@@ -168,13 +199,17 @@ int launch_skinny(const blkq4_gemm_args* a) {
   const auto* Z = static_cast<const uint8_t*>(a->zero_points);
   auto* C = static_cast<uint16_t*>(a->c);
 #define BLKQ4_LAUNCH(ZP_, DEPTH_, NT_)                                                                         \
-  hipLaunchKernelGGL((skinny_mfma_kernel<BS, ZP_, DEPTH_, NT_>), dim3(a->n / (16 * NT_)), block, 0, stream, A, W, \
+  hipLaunchKernelGGL((skinny_mfma_kernel<BS, ZP_, DEPTH_, NT_>), dim3((a->n / 16 + NT_ - 1) / NT_), block, 0, stream, A, W, \
                      S, Z, C, a->m, a->n, a->k)
-  if (Z) {
-    if (a->m <= 4) BLKQ4_LAUNCH(true, 8, 1); else BLKQ4_LAUNCH(true, 4, 2);
-  } else {
-    if (a->m <= 4) BLKQ4_LAUNCH(false, 8, 1); else BLKQ4_LAUNCH(false, 4, 2);
-  }
+  int nt, depth;
+  choose_shape(a->m, a->n, &nt, &depth);
+#define BLKQ4_LAUNCH_ZP(ZP_)                   \
+  if (nt == 1 && depth == 8) BLKQ4_LAUNCH(ZP_, 8, 1); \
+  else if (nt == 1) BLKQ4_LAUNCH(ZP_, 4, 1);   \
+  else if (nt == 2) BLKQ4_LAUNCH(ZP_, 4, 2);   \
+  else BLKQ4_LAUNCH(ZP_, 4, 3)
+  if (Z) { BLKQ4_LAUNCH_ZP(true); } else { BLKQ4_LAUNCH_ZP(false); }
+#undef BLKQ4_LAUNCH_ZP
 #undef BLKQ4_LAUNCH
   return static_cast<int>(hipGetLastError());
 }
@@ -182,7 +217,7 @@ int launch_skinny(const blkq4_gemm_args* a) {
 }  // namespace
 
 extern "C" int blkq4_dev_skinny(const blkq4_gemm_args* a) {
-  if (a->m < 1 || a->m > 16 || (a->n % 32) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
+  if (a->m < 1 || a->m > 16 || (a->n % 16) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
   switch (a->block_size) {
     case 16: return launch_skinny<16>(a);
     case 32: return launch_skinny<32>(a);

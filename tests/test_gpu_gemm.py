@@ -60,9 +60,14 @@ EDGE_CASES = [
     (64, True, 7, 1024, 192), (16, False, 15, 704, 576), (32, True, 17, 96, 192), (64, True, 33, 288, 320),
     (16, True, 65, 544, 256), (32, False, 100, 800, 448), (64, True, 129, 1056, 576), (32, True, 300, 256, 64),
 ]
+# wide N at M <= 16, where the kernel gives a workgroup 1, 2 or 3 column tiles depending on how the
+# tile count fills the chip (258 tiles: 2; 514: 3 with a ragged last workgroup; 1792: 1)
+WIDE_SKINNY_CASES = [
+    (16, True, 12, 4128, 128), (32, True, 8, 8224, 128), (64, False, 3, 8224, 192), (32, False, 5, 28672, 64),
+]
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES)
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
 
