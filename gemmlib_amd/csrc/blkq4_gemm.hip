@@ -47,12 +47,7 @@ namespace {
 
 using namespace blkq4;
 
-constexpr int kWaves = 8;  // two per SIMD
-constexpr int kThreads = 64 * kWaves;
-constexpr int kBN = 32 * kWaves;
 constexpr int kBK = 64;
-constexpr int kStages = 4;    // LDS ring depth
-constexpr int kDistance = 3;  // tiles requested ahead of the one being consumed
 
 // Asynchronous copy: every active lane moves SIZE bytes from global address (base + offset) to
 // LDS[lds_base + lane * SIZE].  lds_base and base are wave-uniform, offset is per lane.  The
@@ -76,42 +71,68 @@ __device__ __forceinline__ void block_barrier() {
 }
 #define BLKQ4_PIN() __builtin_amdgcn_sched_barrier(0)
 
-template <int BS, int RT>
+// MFMA slot (0 .. slots-1) after which copy y of the range [lo, hi) is issued: evenly spread
+constexpr int copy_slot(int y, int lo, int hi, int slots) { return (hi > lo) ? (y - lo) * slots / (hi - lo) : -1; }
+
+// Shape of a workgroup: WM x WN waves, each owning (32*RT) rows x (32*NT) columns (the WM waves of a
+// column group share its packed weights, scales and zero-points), plus PW producer waves that do
+// nothing but issue the async copies.  With PW = 0 the computing waves issue the copies themselves.
+template <int BS, int RT, int NT, int WM, int WN, int PW>
 struct Stage {
-  static constexpr int kBlocks = kBK / BS;                   // quantization block rows per k tile
-  static constexpr int kABytes = 32 * RT * 128;              // [row][8 x 16-byte units, swizzled]
-  static constexpr int kBBytes = kWaves * 1024;              // [wave][lane] 16-byte units
-  static constexpr int kMetaBytes = kWaves * kBlocks * 128;  // [wave][block][64 B scales | 32 B zps | pad]
+  static constexpr int kCopiers = (PW > 0) ? PW : WM * WN;     // waves that share out the copies of a stage
+  static constexpr int kBlocks = kBK / BS;                     // quantization block rows per k tile
+  static constexpr int kABytes = 32 * RT * WM * 128;           // [row][8 x 16-byte units, swizzled]
+  static constexpr int kBBytes = WN * NT * 1024;               // [column group][fragment][lane] 16-byte units
+  static constexpr int kMetaBytes = WN * kBlocks * 256;        // [column group][block][2 fragments][64 B scales | 32 B zps | pad]
   static constexpr int kBytes = kABytes + kBBytes + kMetaBytes;
-  static constexpr int kAOps = (4 * RT + kWaves - 1) / kWaves;  // 8-row activation copies per wave and stage
-  static constexpr int kOps = kAOps + 1 + kBlocks;              // async copies per wave and stage
+  // per copying wave and stage: 8-row activation groups, packed weight fragments, scale / zero-point rows
+  static constexpr int kAOps = (4 * RT * WM + kCopiers - 1) / kCopiers;
+  static constexpr int kBOps = (NT * WN + kCopiers - 1) / kCopiers;
+  static constexpr int kMOps = (WN * kBlocks + kCopiers - 1) / kCopiers;
+  static constexpr int kOps = kAOps + kBOps + kMOps;
+  // ring of k tiles in LDS, requested kDistance tiles ahead of the one being consumed
+  static constexpr int kStages = (4 * kBytes <= 160 * 1024) ? 4 : 3;
+  static constexpr int kDistance = kStages - 1;  // the slot being refilled is the one nobody reads
 };
 
-template <int BS, bool HAS_ZP, int RT>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_mfma_kernel(
-    const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ S,
-    const uint8_t* __restrict__ Z, uint16_t* __restrict__ C, int M, int N, int K, int m_tiles) {
-  using St = Stage<BS, RT>;
+template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW>
+__global__ __launch_bounds__(64 * (WM * WN + PW))
+    __attribute__((amdgpu_waves_per_eu((WM * WN + PW) / 4, (WM * WN + PW) / 4))) void gemm_mfma_kernel(
+        const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ S,
+        const uint8_t* __restrict__ Z, uint16_t* __restrict__ C, int M, int N, int K, int m_tiles) {
+  using St = Stage<BS, RT, NT, WM, WN, PW>;
+  constexpr int kComputeWaves = WM * WN;
+  constexpr int kCopiers = St::kCopiers;
+  static_assert((WM * WN + PW) % 4 == 0, "whole waves per SIMD");
   constexpr int kBlocks = St::kBlocks;
   constexpr int kOps = St::kOps;
+  constexpr int kStages = St::kStages;
+  constexpr int kDistance = St::kDistance;
+  constexpr int kBN = 32 * NT * WN;
+  constexpr int kBM = 32 * RT * WM;
   constexpr int kMeta = (BS == 16) ? 2 : 1;  // quantization blocks inside a lane's 32-deep unit
+  constexpr int kMfmas = RT * NT;            // MFMAs of one 16-deep k step
   static_assert(kStages * St::kBytes <= 160 * 1024, "LDS ring does not fit");
-  static_assert(kDistance == kStages - 1, "the stage being refilled must be the one nobody reads");
+  static_assert(NT == 1 || NT == 2, "the scale / zero-point copy covers at most two fragments");
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kStages * St::kBytes];
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = (wave / WN) % WM;  // position of the wave's tile inside the workgroup tile
+  const int wn = wave % WN;
+  const int cw = (PW > 0) ? max(wave - kComputeWaves, 0) : wave;  // index among the copying waves
   const int lane = tid & 63;
   const int i = lane & 31;  // row of an activation fragment / column of a weight fragment
   const int h = lane >> 5;  // which 32-deep half of the 64-deep k tile this lane covers
 
   const int bm = blockIdx.x % m_tiles;
   const int bn = blockIdx.x / m_tiles;
-  const int m0 = bm * (32 * RT);
-  const int nw0 = bn * kBN + wave * 32;
-  // N is a multiple of 32, so 32-column tiles are whole; a tile past the end re-reads the last one
-  const bool tile_ok = nw0 < N;
-  const int nbase = min(nw0, N - 32);
+  const int m0 = bm * kBM;
+  const int nw0 = bn * kBN + wn * (32 * NT);
+  // N is a multiple of 32, so 32-column fragments are whole; a fragment past the end re-reads the last one
+  int nbase[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) nbase[t] = min(nw0 + 32 * t, N - 32);
   const int KT = K / kBK;
 
   // ---- per-lane byte offsets of the async copies inside k tile 0 ----
@@ -120,111 +141,208 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   uint32_t a_dst[kAOps];  // LDS byte offset of the 8-row group inside the stage
 #pragma unroll
   for (int p = 0; p < kAOps; ++p) {
-    // 4*RT groups of 8 rows are shared out over the waves; with fewer groups than waves the extra
-    // waves copy a group a second time (same bytes to the same place) so that every wave has the
-    // same number of copies in flight
-    const int group = (kWaves * p + wave) % (4 * RT);
+    // 4*RT*WM groups of 8 rows are shared out over the copying waves; when the division leaves a
+    // remainder some waves copy a group a second time (same bytes to the same place) so that every
+    // wave has the same number of copies in flight
+    const int group = (kCopiers * p + cw) % (4 * RT * WM);
     a_dst[p] = group * 1024;
     const int row = 8 * group + (lane >> 3);  // row inside the tile
     const int col = (lane & 7) ^ ((row >> 1) & 7);     // logical 16-byte column this lane fetches
     a_off[p] = static_cast<uint32_t>(min(m0 + row, M - 1)) * (static_cast<uint32_t>(K) * 2u) + col * 16;
   }
-  const uint32_t b_off = (static_cast<uint32_t>(h) * N + nbase + i) * 16u;
+  // the NT*WN weight fragments of the workgroup tile, shared out the same way
+  constexpr int kBOps = St::kBOps;
+  uint32_t b_off[kBOps];
+  uint32_t b_dst[kBOps];
+#pragma unroll
+  for (int p = 0; p < kBOps; ++p) {
+    const int f = (kCopiers * p + cw) % (NT * WN);  // fragment f: column group f / NT, fragment f % NT
+    const int nb = min(bn * kBN + 32 * f, N - 32);
+    b_off[p] = (static_cast<uint32_t>(h) * N + nb + i) * 16u;
+    b_dst[p] = St::kABytes + f * 1024;
+  }
   const uint32_t b_stride = static_cast<uint32_t>(N) * 32u;  // two 32-deep units per k tile
-  // meta: lanes 0..15 fetch 2 scales each, lanes 16..23 fetch 4 zero-points each
-  const bool meta_active = HAS_ZP ? (lane < 24) : (lane < 16);
-  const bool meta_is_scale = lane < 16 || !HAS_ZP;
-  const uint8_t* meta_ptr = (meta_is_scale ? S + static_cast<size_t>(nbase + 2 * (lane & 15)) * 2
-                                           : Z + (nbase + 4 * (lane & 7)));
+  // meta: one copy per (column group, block row).  Per 32-lane half (= fragment): lanes 0..15 fetch 2
+  // scales each, lanes 16..23 fetch 4 zero-points each.  The copy lands at 4 * lane inside a 256-byte
+  // row, so the lanes with nothing to fetch write into padding; they re-read a scale so that the copy
+  // needs no branch.
+  constexpr int kMOps = St::kMOps;
+  const bool meta_is_scale = i < 16 || i >= 24 || !HAS_ZP;
   const uint32_t meta_row_bytes = meta_is_scale ? static_cast<uint32_t>(N) * 2u : static_cast<uint32_t>(N);
+  const uint8_t* meta_ptr[kMOps];
+  uint32_t meta_dst[kMOps];
+#pragma unroll
+  for (int p = 0; p < kMOps; ++p) {
+    const int idx = (kCopiers * p + cw) % (WN * kBlocks);  // column group idx / kBlocks, block row idx % kBlocks
+    const int nb = min(bn * kBN + (idx / kBlocks) * (32 * NT) + ((NT == 2) ? 32 * h : 0), N - 32);
+    meta_ptr[p] = (meta_is_scale ? S + static_cast<size_t>(nb + 2 * (i & 15)) * 2 : Z + (nb + 4 * (i & 7))) +
+                  static_cast<size_t>(idx % kBlocks) * meta_row_bytes;
+    meta_dst[p] = St::kABytes + St::kBBytes + idx * 256;
+  }
 
   const uint32_t lds0 = static_cast<uint32_t>(
       reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)(&lds[0])));  // LDS byte address
 
   // Async copy number q (0 .. kOps-1) of k tile `tile_` into ring slot `stage_`:
-  // q < kAOps: 8 activation rows; q == kAOps: this wave's packed weights; above: one scale/zero-point row.
+  // q < kAOps: 8 activation rows; the next kBOps: packed weight fragments; above: one
+  // scale/zero-point row (all fragments of the column group).
 #define BLKQ4_COPY_OP(q_, tile_, stage_)                                                                  \
   {                                                                                                       \
     const uint32_t sbase_ = lds0 + (stage_) * St::kBytes;                                                 \
     if ((q_) < kAOps) {                                                                                   \
       async_copy_16(sbase_ + a_dst[(q_) < kAOps ? (q_) : 0], A + static_cast<size_t>(tile_) * 128,       \
                     a_off[(q_) < kAOps ? (q_) : 0]);                                                      \
-    } else if ((q_) == kAOps) {                                                                           \
-      async_copy_16(sbase_ + St::kABytes + wave * 1024, W + static_cast<size_t>(tile_) * b_stride, b_off); \
-    } else if (meta_active) {                                                                             \
-      async_copy_4_flat(sbase_ + St::kABytes + St::kBBytes + (wave * kBlocks + ((q_) - kAOps - 1)) * 128,    \
-                        meta_ptr + static_cast<size_t>((tile_) * kBlocks + ((q_) - kAOps - 1)) * meta_row_bytes); \
+    } else if ((q_) < kAOps + kBOps) {                                                                    \
+      const int p_ = ((q_) >= kAOps && (q_) < kAOps + kBOps) ? (q_) - kAOps : 0;                           \
+      async_copy_16(sbase_ + b_dst[p_], W + static_cast<size_t>(tile_) * b_stride, b_off[p_]);            \
+    } else {                                                                                              \
+      const int p_ = ((q_) >= kAOps + kBOps) ? (q_) - kAOps - kBOps : 0;                                   \
+      async_copy_4_flat(sbase_ + meta_dst[p_],                                                            \
+                        meta_ptr[p_] + static_cast<size_t>(tile_) * (kBlocks * meta_row_bytes));           \
     }                                                                                                     \
   }
 
-  float16_t acc[RT];
+  if (PW > 0 && wave >= kComputeWaves) {
+    // Producer wave: requests k tiles kDistance ahead and meets the computing waves at their barrier
+    // once per tile, after its copies for the tile they are about to start reading have landed.
+#pragma unroll
+    for (int s = 0; s < kDistance; ++s) {
+#pragma unroll
+      for (int q = 0; q < kOps; ++q) BLKQ4_COPY_OP(q, min(s, KT - 1), s);
+    }
+    wait_vmcnt<(kDistance - 1) * kOps>();
+    block_barrier();
+    for (int kt = 0; kt < KT; ++kt) {
+      // tile kt+1 must have landed: everything but the kDistance-2 newest groups (near the end
+      // fewer groups than that are in flight, then wait for all of them)
+      if (kt + kDistance <= KT) {
+        wait_vmcnt<(kDistance - 2) * kOps>();
+      } else {
+        wait_vmcnt<0>();
+      }
+      block_barrier();  // also: nobody reads the slot of tile kt-1 any more
+      if (kt + kDistance < KT) {
+        const int stage = (kt + kDistance) % kStages;
+#pragma unroll
+        for (int q = 0; q < kOps; ++q) BLKQ4_COPY_OP(q, kt + kDistance, stage);
+      }
+    }
+    wait_vmcnt<0>();
+    return;
+  }
+
+  float16_t acc[RT][NT];
 #pragma unroll
   for (int r = 0; r < RT; ++r)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[r][e] = 0.f;
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[r][t][e] = 0.f;
 
   // ---- prologue: request tiles 0 .. kDistance-1, publish tile 0 ----
+  // (when a tile's copies are spread over four steps, the second half of the last of these tiles is
+  // issued by steps 0 and 1 of the first loop iteration, like every later one)
+  constexpr int kPrologueLast = (St::kStages >= 4) ? (kOps * 2 / 4) : kOps;
+  if (PW == 0) {
 #pragma unroll
-  for (int s = 0; s < kDistance; ++s) {
+    for (int s = 0; s < kDistance; ++s) {
 #pragma unroll
-    for (int q = 0; q < kOps; ++q) BLKQ4_COPY_OP(q, min(s, KT - 1), s);
+      for (int q = 0; q < ((s == kDistance - 1) ? kPrologueLast : kOps); ++q) BLKQ4_COPY_OP(q, min(s, KT - 1), s);
+    }
+    wait_vmcnt<(kDistance - 2) * kOps + kPrologueLast>();
   }
-  wait_vmcnt<(kDistance - 1) * kOps>();
   block_barrier();
 
   // ---- LDS byte offsets of this lane's reads inside a stage ----
   uint32_t a_rd[4];  // activation fragment of step j, row tile 0 (row tile r is 4096 bytes further)
 #pragma unroll
-  for (int j = 0; j < 4; ++j) a_rd[j] = static_cast<uint32_t>(i) * 128u + (((4 * h + j) ^ ((i >> 1) & 7)) * 16u);
-  const uint32_t b_rd = St::kABytes + wave * 1024 + lane * 16;
-  const uint32_t m_rd = St::kABytes + St::kBBytes + wave * kBlocks * 128;
+  for (int j = 0; j < 4; ++j) {
+    a_rd[j] = static_cast<uint32_t>(wm * (32 * RT) + i) * 128u + (((4 * h + j) ^ ((i >> 1) & 7)) * 16u);
+  }
+  const uint32_t b_rd = St::kABytes + wn * (NT * 1024) + lane * 16;
+  const uint32_t m_rd = St::kABytes + St::kBBytes + wn * kBlocks * 256;
 
   const DequantMasks masks = DequantMasks::make();
 
-#define BLKQ4_READ_A(dst_, stage_ptr_, j_)                                                   \
-  _Pragma("unroll") for (int r = 0; r < RT; ++r)(dst_)[r] =                                  \
-      as_half8(*reinterpret_cast<const uint4*>((stage_ptr_) + a_rd[j_] + r * 4096))
 #define BLKQ4_READ_A1(dst_, stage_ptr_, j_, r_) \
   (dst_)[r_] = as_half8(*reinterpret_cast<const uint4*>((stage_ptr_) + a_rd[j_] + (r_) * 4096))
+  // packed words, scales and zero-points of all the wave's fragments for one k tile
 #define BLKQ4_READ_B(words_, dc_, stage_ptr_)                                                \
-  {                                                                                          \
-    const uint4 u_ = *reinterpret_cast<const uint4*>((stage_ptr_) + b_rd);                   \
-    (words_)[0] = u_.x;                                                                      \
-    (words_)[1] = u_.y;                                                                      \
-    (words_)[2] = u_.z;                                                                      \
-    (words_)[3] = u_.w;                                                                      \
+  _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                           \
+    const uint4 u_ = *reinterpret_cast<const uint4*>((stage_ptr_) + b_rd + t * 1024);        \
+    (words_)[t][0] = u_.x;                                                                   \
+    (words_)[t][1] = u_.y;                                                                   \
+    (words_)[t][2] = u_.z;                                                                   \
+    (words_)[t][3] = u_.w;                                                                   \
     _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                      \
       const int blk_ = (BS == 64) ? 0 : (BS == 32) ? h : (2 * h + q);                        \
-      const uint8_t* mb_ = (stage_ptr_) + m_rd + blk_ * 128;                                 \
-      (dc_##_sc)[q] = *reinterpret_cast<const uint16_t*>(mb_ + i * 2);                       \
-      (dc_##_zp)[q] = HAS_ZP ? static_cast<uint32_t>(mb_[64 + i]) : 8u;                      \
+      const uint8_t* mb_ = (stage_ptr_) + m_rd + (blk_ * 2 + t) * 128;                       \
+      (dc_##_sc)[t][q] = *reinterpret_cast<const uint16_t*>(mb_ + i * 2);                    \
+      (dc_##_zp)[t][q] = HAS_ZP ? static_cast<uint32_t>(mb_[64 + i]) : 8u;                   \
     }                                                                                        \
   }
-  // piece p (0..3) of the conversion of `word_` into weight fragment slot `dst_`
-#define BLKQ4_PIECE(dst_, word_, dc_, p_) \
-  wp[dst_][p_] = dequant_pair(((p_) >= 2) ? ((word_) >> 8) : (word_), (p_), (dc_), masks)
-#define BLKQ4_WFRAG(slot_) \
-  __builtin_bit_cast(half8_t, half2x4_t{wp[slot_][0], wp[slot_][1], wp[slot_][2], wp[slot_][3]})
+#define BLKQ4_MAKE_CONSTS(dc_)                            \
+  _Pragma("unroll") for (int t = 0; t < NT; ++t)          \
+  _Pragma("unroll") for (int q = 0; q < kMeta; ++q)(dc_)[t][q] = make_dequant_consts((dc_##_sc)[t][q], (dc_##_zp)[t][q])
+  // piece x (0 .. 4*NT-1) of the conversion of word `w_` of every fragment into fragment buffer `dst_`:
+  // piece x is fp16 pair x % 4 of fragment x / 4
+#define BLKQ4_PIECE(dst_, words_, w_, dc_, q_, x_)                                                         \
+  wp[dst_][(x_) / 4][(x_) % 4] =                                                                           \
+      dequant_pair((((x_) % 4) >= 2) ? ((words_)[(x_) / 4][w_] >> 8) : (words_)[(x_) / 4][w_], (x_) % 4, \
+                   (dc_)[(x_) / 4][q_], masks)
+#define BLKQ4_WFRAG(slot_, t_) \
+  __builtin_bit_cast(half8_t, half2x4_t{wp[slot_][t_][0], wp[slot_][t_][1], wp[slot_][t_][2], wp[slot_][t_][3]})
 
   struct half2x4_t {
     half2_t a, b, c, d;
   };
 
-  half8_t af[2][RT];   // activation fragments, double buffered over the k steps
-  half2_t wp[2][4];    // weight fragment (4 fp16 pairs), double buffered
-  uint32_t words[4], nwords[4];
-  uint32_t dc_sc[kMeta], dc_zp[kMeta], ndc_sc[kMeta], ndc_zp[kMeta];
-  DequantConsts dc[kMeta], ndc[kMeta];
+  half8_t af[2][RT];      // activation fragments, double buffered over the k steps
+  half2_t wp[2][NT][4];   // weight fragments (4 fp16 pairs each), double buffered
+  uint32_t words[NT][4], nwords[NT][4];
+  uint32_t dc_sc[NT][kMeta], dc_zp[NT][kMeta], ndc_sc[NT][kMeta], ndc_zp[NT][kMeta];
+  DequantConsts dc[NT][kMeta], ndc[NT][kMeta];
 
   {
     const uint8_t* s0 = lds;
     BLKQ4_READ_B(words, dc, s0);
+    BLKQ4_MAKE_CONSTS(dc);
 #pragma unroll
-    for (int q = 0; q < kMeta; ++q) dc[q] = make_dequant_consts(dc_sc[q], dc_zp[q]);
-    BLKQ4_READ_A(af[0], s0, 0);
+    for (int r = 0; r < RT; ++r) BLKQ4_READ_A1(af[0], s0, 0, r);
 #pragma unroll
-    for (int p = 0; p < 4; ++p) BLKQ4_PIECE(0, words[0], dc[0], p);
+    for (int x = 0; x < 4 * NT; ++x) BLKQ4_PIECE(0, words, 0, dc, 0, x);
   }
+
+  // One 16-deep k step: RT*NT MFMAs on fragment buffers `cur_`; in their shadow the LDS reads of the
+  // next step's activation fragments (from `nstage_`, step `nj_`), the conversion of the next weight
+  // fragments (word `nw_` of `nwords_`) and, in the second half of a tile, the async copies
+  // lo_ .. hi_-1 of k tile ctile_ (into ring slot cstage_), spread evenly over the step.
+#define BLKQ4_STEP(cur_, nstage_, nj_, nwords_, nw_, ndc_, nq_, lo_, hi_, ctile_, cstage_)         \
+  {                                                                                                \
+    half8_t wf_[NT];                                                                               \
+    _Pragma("unroll") for (int t = 0; t < NT; ++t) wf_[t] = BLKQ4_WFRAG(cur_, t);                  \
+    _Pragma("unroll") for (int r = 0; r < RT; ++r) {                                               \
+      _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                             \
+        const int x_ = r * NT + t;                                                                 \
+        acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[t], af[cur_][r], acc[r][t], 0, 0, 0); \
+        if (t == NT - 1) BLKQ4_READ_A1(af[1 - (cur_)], nstage_, nj_, r);                           \
+        _Pragma("unroll") for (int y = x_ * kPiecesPerMfma; y < (x_ + 1) * kPiecesPerMfma; ++y) {  \
+          if (y < 4 * NT) BLKQ4_PIECE(1 - (cur_), nwords_, nw_, ndc_, nq_, y);                     \
+        }                                                                                          \
+        _Pragma("unroll") for (int y = (lo_); y < (hi_); ++y) {                                    \
+          if (copy_slot(y, lo_, hi_, kMfmas) == x_) BLKQ4_COPY_OP(y, ctile_, cstage_);             \
+        }                                                                                          \
+        BLKQ4_PIN();                                                                               \
+      }                                                                                            \
+    }                                                                                              \
+  }
+  constexpr int kPiecesPerMfma = (4 * NT + kMfmas - 1) / kMfmas;
+  // The copies of one k tile are issued over the four steps that follow the barrier which frees
+  // their ring slot (two steps when the ring has only three slots and the tile is needed sooner).
+  constexpr int kCopySteps = (PW > 0) ? 0 : (kStages >= 4) ? 4 : 2;  // 0: the producer waves copy
+  constexpr int kCut1 = (kCopySteps == 0) ? 0 : kOps * 1 / (kCopySteps == 0 ? 1 : kCopySteps);
+  constexpr int kCut2 = (kCopySteps == 4) ? kOps * 2 / 4 : (kCopySteps == 2) ? kOps : 0;
+  constexpr int kCut3 = kOps * 3 / 4;
 
   for (int kt = 0; kt < KT; ++kt) {
     const int stage = kt % kStages;
@@ -232,111 +350,72 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const uint8_t* sn = lds + ((kt + 1) % kStages) * St::kBytes;          // tile kt + 1
     const int copy_tile = min(kt + kDistance, KT - 1);                    // clamped: re-fetches the last tile
     const int copy_stage = (kt + kDistance) % kStages;
+    const int late_tile = min(kt + kDistance - 1, KT - 1);                // the group begun in the previous tile
+    const int late_stage = (kt + kDistance - 1) % kStages;
     BLKQ4_PIN();
 
-    // ---------------- step 0: uses af[0] / wp[0]; prepares step 1 ----------------
-    {
-      const half8_t wf = BLKQ4_WFRAG(0);
-#pragma unroll
-      for (int r = 0; r < RT; ++r) {
-        acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf, af[0][r], acc[r], 0, 0, 0);
-        BLKQ4_READ_A1(af[1], sa, 1, r);
-        if (r < 4) BLKQ4_PIECE(1, words[1], dc[0], r);
-        BLKQ4_PIN();
-      }
-#pragma unroll
-      for (int p = RT; p < 4; ++p) BLKQ4_PIECE(1, words[1], dc[0], p);
-    }
-    // ---------------- step 1: uses af[1] / wp[1]; prepares step 2 ----------------
-    {
-      const half8_t wf = BLKQ4_WFRAG(1);
-#pragma unroll
-      for (int r = 0; r < RT; ++r) {
-        acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf, af[1][r], acc[r], 0, 0, 0);
-        BLKQ4_READ_A1(af[0], sa, 2, r);
-        if (r < 4) BLKQ4_PIECE(0, words[2], dc[kMeta - 1], r);
-        BLKQ4_PIN();
-      }
-#pragma unroll
-      for (int p = RT; p < 4; ++p) BLKQ4_PIECE(0, words[2], dc[kMeta - 1], p);
-    }
+    // step 0: uses buffers 0; prepares step 1
+    BLKQ4_STEP(0, sa, 1, words, 1, dc, 0, (kCopySteps == 4 ? kCut2 : 0), (kCopySteps == 4 ? kCut3 : 0), late_tile, late_stage);
+    // step 1: uses buffers 1; prepares step 2
+    BLKQ4_STEP(1, sa, 2, words, 2, dc, kMeta - 1, (kCopySteps == 4 ? kCut3 : 0), (kCopySteps == 4 ? kOps : 0), late_tile, late_stage);
     // publish tile kt+1: this wave's copies for it have landed, then everybody's
-    wait_vmcnt<kOps>();
+    if (PW == 0) wait_vmcnt<(kDistance - 2) * kOps>();
     block_barrier();
-    // ---------------- step 2: uses af[0] / wp[0]; prepares step 3, reads next tile's weights ----
+    // step 2: uses buffers 0; prepares step 3, reads the next tile's weights, starts the copies
     BLKQ4_READ_B(nwords, ndc, sn);
     BLKQ4_PIN();
-    {
-      const half8_t wf = BLKQ4_WFRAG(0);
-#pragma unroll
-      for (int r = 0; r < RT; ++r) {
-        acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf, af[0][r], acc[r], 0, 0, 0);
-        BLKQ4_READ_A1(af[1], sa, 3, r);
-        if (r < 4) BLKQ4_PIECE(1, words[3], dc[kMeta - 1], r);
-        if (r < kOps) BLKQ4_COPY_OP(r, copy_tile, copy_stage);
-        BLKQ4_PIN();
-      }
-#pragma unroll
-      for (int p = RT; p < 4; ++p) BLKQ4_PIECE(1, words[3], dc[kMeta - 1], p);
-    }
-    // ---------------- step 3: uses af[1] / wp[1]; prepares step 0 of tile kt+1 ----------------
-#pragma unroll
-    for (int q = 0; q < kMeta; ++q) ndc[q] = make_dequant_consts(ndc_sc[q], ndc_zp[q]);
+    BLKQ4_STEP(0, sa, 3, words, 3, dc, kMeta - 1, 0, kCut1, copy_tile, copy_stage);
+    // step 3: uses buffers 1; prepares step 0 of tile kt+1, finishes the copies
+    BLKQ4_MAKE_CONSTS(ndc);
     BLKQ4_PIN();
-    {
-      const half8_t wf = BLKQ4_WFRAG(1);
+    BLKQ4_STEP(1, sn, 0, nwords, 0, ndc, 0, kCut1, kCut2, copy_tile, copy_stage);
 #pragma unroll
-      for (int r = 0; r < RT; ++r) {
-        acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf, af[1][r], acc[r], 0, 0, 0);
-        BLKQ4_READ_A1(af[0], sn, 0, r);
-        if (r < 4) BLKQ4_PIECE(0, nwords[0], ndc[0], r);
-        if (RT + r < kOps) BLKQ4_COPY_OP(RT + r, copy_tile, copy_stage);
-        BLKQ4_PIN();
-      }
+    for (int t = 0; t < NT; ++t) {
 #pragma unroll
-      for (int p = RT; p < 4; ++p) BLKQ4_PIECE(0, nwords[0], ndc[0], p);
+      for (int j = 0; j < 4; ++j) words[t][j] = nwords[t][j];
 #pragma unroll
-      for (int q = 2 * RT; q < kOps; ++q) BLKQ4_COPY_OP(q, copy_tile, copy_stage);
+      for (int q = 0; q < kMeta; ++q) dc[t][q] = ndc[t][q];
     }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) words[j] = nwords[j];
-#pragma unroll
-    for (int q = 0; q < kMeta; ++q) dc[q] = ndc[q];
   }
-  wait_vmcnt<0>();  // the clamped re-fetches of the last tile are still in flight
+  if (PW == 0) wait_vmcnt<0>();  // the clamped re-fetches of the last tile are still in flight
 #undef BLKQ4_COPY_OP
-#undef BLKQ4_READ_A
 #undef BLKQ4_READ_A1
 #undef BLKQ4_READ_B
+#undef BLKQ4_MAKE_CONSTS
 #undef BLKQ4_PIECE
 #undef BLKQ4_WFRAG
+#undef BLKQ4_STEP
 
-  // Epilogue.  Accumulator element 4*g + e of lane (i, h) is output row m0 + 32*r + i and column
-  // nw0 + 8*g + 4*h + e: four consecutive columns -> one 8-byte store.
-  if (!tile_ok) return;
+  // Epilogue.  Accumulator element 4*g + e of lane (i, h), fragment t, is output row m0 + 32*r + i and
+  // column nw0 + 32*t + 8*g + 4*h + e: four consecutive columns -> one 8-byte store.
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
-    const int m = m0 + 32 * r + i;
+    const int m = m0 + wm * (32 * RT) + 32 * r + i;
     if (m >= M) continue;
-    uint16_t* crow = C + static_cast<size_t>(m) * N + nw0 + 4 * h;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const uint32_t lo = float_to_half_bits(acc[r][4 * g + 0]) |
-                          (static_cast<uint32_t>(float_to_half_bits(acc[r][4 * g + 1])) << 16);
-      const uint32_t hi = float_to_half_bits(acc[r][4 * g + 2]) |
-                          (static_cast<uint32_t>(float_to_half_bits(acc[r][4 * g + 3])) << 16);
-      *reinterpret_cast<uint2*>(crow + 8 * g) = make_uint2(lo, hi);
+    for (int t = 0; t < NT; ++t) {
+      if (nw0 + 32 * t >= N) continue;
+      uint16_t* crow = C + static_cast<size_t>(m) * N + nw0 + 32 * t + 4 * h;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const uint32_t lo = float_to_half_bits(acc[r][t][4 * g + 0]) |
+                            (static_cast<uint32_t>(float_to_half_bits(acc[r][t][4 * g + 1])) << 16);
+        const uint32_t hi = float_to_half_bits(acc[r][t][4 * g + 2]) |
+                            (static_cast<uint32_t>(float_to_half_bits(acc[r][t][4 * g + 3])) << 16);
+        *reinterpret_cast<uint2*>(crow + 8 * g) = make_uint2(lo, hi);
+      }
     }
   }
 }
 
-template <int BS, bool HAS_ZP, int RT>
+template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW>
 int launch_one(const blkq4_gemm_args* a) {
-  constexpr int BM = 32 * RT;
+  constexpr int BM = 32 * RT * WM;
+  constexpr int kBN = 32 * NT * WN;
   const int m_tiles = (a->m + BM - 1) / BM;
   const int n_tiles = (a->n + kBN - 1) / kBN;
   const dim3 grid(static_cast<unsigned>(m_tiles) * n_tiles);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BS, HAS_ZP, RT>), grid, dim3(kThreads), 0,
+  hipLaunchKernelGGL((gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW>), grid, dim3(64 * (WM * WN + PW)), 0,
                      static_cast<hipStream_t>(a->stream), static_cast<const uint8_t*>(a->a),
                      static_cast<const uint8_t*>(a->packed_w), static_cast<const uint8_t*>(a->scales),
                      static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c), a->m, a->n,
@@ -347,9 +426,13 @@ int launch_one(const blkq4_gemm_args* a) {
 template <int BS, bool HAS_ZP>
 int launch_rt(const blkq4_gemm_args* a) {
   // rows per workgroup: 128 unless the whole problem is shorter
-  if (a->m <= 32) return launch_one<BS, HAS_ZP, 1>(a);
-  if (a->m <= 64) return launch_one<BS, HAS_ZP, 2>(a);
-  return launch_one<BS, HAS_ZP, 4>(a);
+  if (a->m <= 32) return launch_one<BS, HAS_ZP, 1, 1, 1, 8, 0>(a);
+  if (a->m <= 64) return launch_one<BS, HAS_ZP, 2, 1, 1, 8, 0>(a);
+#ifdef BLKQ4_GEMM_SHAPE
+  return launch_one<BS, HAS_ZP, BLKQ4_GEMM_SHAPE>(a);
+#else
+  return launch_one<BS, HAS_ZP, 4, 2, 1, 4, 4>(a);
+#endif
 }
 
 template <int BS>
