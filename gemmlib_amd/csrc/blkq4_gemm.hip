@@ -42,34 +42,13 @@
 
 #include "blkq4_dequant.h"
 #include "blkq4_device.h"
+#include "blkq4_gemm_common.h"
 
 namespace {
 
 using namespace blkq4;
 
 constexpr int kBK = 64;
-
-// Asynchronous copy: every active lane moves SIZE bytes from global address (base + offset) to
-// LDS[lds_base + lane * SIZE].  lds_base and base are wave-uniform, offset is per lane.  The
-// compiler does not see the LDS write (it is ordered by hand with wait_vmcnt + s_barrier below).
-__device__ __forceinline__ void async_copy_16(uint32_t lds_base, const void* base, uint32_t offset) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base)
-               : "memory");
-}
-__device__ __forceinline__ void async_copy_4_flat(uint32_t lds_base, const void* gptr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-// s_barrier that the compiler may not move LDS accesses across, in either direction
-__device__ __forceinline__ void block_barrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-#define BLKQ4_PIN() __builtin_amdgcn_sched_barrier(0)
 
 // MFMA slot (0 .. slots-1) after which copy y of the range [lo, hi) is issued: evenly spread
 constexpr int copy_slot(int y, int lo, int hi, int slots) { return (hi > lo) ? (y - lo) * slots / (hi - lo) : -1; }
@@ -425,12 +404,19 @@ int launch_one(const blkq4_gemm_args* a) {
 
 template <int BS, bool HAS_ZP>
 int launch_rt(const blkq4_gemm_args* a) {
-  // rows per workgroup: 128 unless the whole problem is shorter
+  // rows per workgroup: no more than the problem has
   if (a->m <= 32) return launch_one<BS, HAS_ZP, 1, 1, 1, 8, 0>(a);
   if (a->m <= 64) return launch_one<BS, HAS_ZP, 2, 1, 1, 8, 0>(a);
 #ifdef BLKQ4_GEMM_SHAPE
   return launch_one<BS, HAS_ZP, BLKQ4_GEMM_SHAPE>(a);
 #else
+  // Problems with at least one 256 x 256 tile per compute unit: four waves of 256 x 64 each, the
+  // fewest conversion instructions per MFMA (every register of a SIMD belongs to one wave, which
+  // leaves no room for producer waves).  Smaller ones: 128 x 256 tiles, four waves of 128 x 64 plus
+  // four producer waves.
+  constexpr int kComputeUnits = 256;
+  const long tiles = static_cast<long>((a->m + 255) / 256) * ((a->n + 255) / 256);
+  if (tiles >= kComputeUnits) return launch_one<BS, HAS_ZP, 8, 2, 1, 4, 0>(a);
   return launch_one<BS, HAS_ZP, 4, 2, 1, 4, 4>(a);
 #endif
 }

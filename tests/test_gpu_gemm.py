@@ -62,12 +62,14 @@ EDGE_CASES = [
 ]
 # wide N at M <= 16, where the kernel gives a workgroup 1, 2 or 3 column tiles depending on how the
 # tile count fills the chip (258 tiles: 2; 514: 3 with a ragged last workgroup; 1792: 1)
+# shapes with at least 256 tiles of 256 x 256, which take the kernel variant with 256-row waves
+LARGE_TILE_CASES = [(64, True, 4096, 4096, 128), (16, True, 4000, 4128, 64), (32, False, 4096, 4096, 192)]
 WIDE_SKINNY_CASES = [
     (16, True, 12, 4128, 128), (32, True, 8, 8224, 128), (64, False, 3, 8224, 192), (32, False, 5, 28672, 64),
 ]
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES)
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
 
