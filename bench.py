@@ -176,6 +176,27 @@ def bench_prepack(torch, capi, device, steps, warmup):
     }
 
 
+def bench_copy(torch, capi, device, steps, warmup):
+    """A plain copy of known size (the library's layout conversion of a packed weight buffer reads
+    every byte once and writes every byte once): the reference that hardware traffic counters are
+    scaled by.  Not part of the default run."""
+    rows, cols = 16384, 16384
+    nbytes = rows * cols // 2
+    src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=device)
+    dst = torch.empty_like(src)
+    launches = [lambda: capi.repack(True, rows, cols, src, dst)]
+    steps = max(10, steps // 10)
+    wall, evt, mode = timed_region(torch, launches, steps, max(2, warmup // 10))
+    per = evt / steps
+    ach = 2 * nbytes / per / 1e9
+    return {
+        "workload": "copy reference: repack of a 16384x16384 packed buffer (128 MiB read + 128 MiB written)",
+        "value": round(ach, 3), "unit": "GB/s", "ms_per_step": round(wall / steps * 1e3, 6),
+        "kernel_us": round(per * 1e6, 3), "timing": mode, "bytes": 2 * nbytes, "read_bytes": nbytes,
+        "write_bytes": nbytes,
+    }
+
+
 def cpu_baseline(name, a_dev, w_host, target_seconds=12.0):
     """The oracle's dequantize + GEMM on a bounded sample of rows of the same workload."""
     import numpy as np
@@ -235,6 +256,8 @@ def main(argv=None) -> int:
     for name in wanted:
         if name == "prepack":
             results["C5_prepack"] = bench_prepack(torch, capi, device, args.steps, args.warmup)
+        elif name == "copy":
+            results["copy"] = bench_copy(torch, capi, device, args.steps, args.warmup)
         else:
             res, problem = bench_gemm(torch, capi, name, device, args.steps, args.warmup)
             results[name] = res

@@ -33,6 +33,14 @@ __device__ __forceinline__ uint16_t float_to_half_bits(float f) {
   return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));  // v_cvt_f16_f32, round to nearest even
 }
 
+// roundf (halves away from zero) for 0 <= x <= 15 as one add and one truncating conversion.  The
+// constant is the largest float below 0.5: x + c lands on the next integer exactly when
+// x - floor(x) >= 0.5 (checked against roundf for every float in [0, 16]); adding 0.5 itself would
+// round 0.49999997 up to 1.
+__device__ __forceinline__ uint32_t round_0_to_15(float x) {
+  return static_cast<uint32_t>(__fadd_rn(x, 0.49999997f));
+}
+
 // nibble position of weight t (0..7) inside its 32-bit word
 __device__ __forceinline__ constexpr int nibble_shift(int t) { return 4 * ((t >> 1) + 4 * (t & 1)); }
 
@@ -87,23 +95,20 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
       v[2 * i] = half_bits_to_float(words[i] & 0xffffu);
       v[2 * i + 1] = half_bits_to_float(words[i] >> 16);
     }
-    // range over this lane's 8 weights, ascending k, strict compares (first of equal values wins)
+    // Range of the block: this lane's 8 weights, then the lanes that share the block.  The reference
+    // scans in ascending k with strict compares, i.e. among equal values the first wins; that only
+    // shows when +0 and -0 tie, and only matters for an all-zero block without zero-points, whose
+    // scale takes the sign of the block's first weight: handled below from that weight itself.
     float mn = v[0], mx = v[0];
 #pragma unroll
     for (int i = 1; i < 8; ++i) {
-      if (v[i] < mn) mn = v[i];
-      if (v[i] > mx) mx = v[i];
+      mn = fminf(mn, v[i]);
+      mx = fmaxf(mx, v[i]);
     }
-    // ... and across the lanes of the block; "lower" holds the smaller k, which must win ties
 #pragma unroll
     for (int mask = 1; mask < kLanesPerBlock; mask <<= 1) {
-      const float omn = __shfl_xor(mn, mask);
-      const float omx = __shfl_xor(mx, mask);
-      const bool lower = (lane & mask) == 0;
-      const float lo_mn = lower ? mn : omn, hi_mn = lower ? omn : mn;
-      const float lo_mx = lower ? mx : omx, hi_mx = lower ? omx : mx;
-      mn = (hi_mn < lo_mn) ? hi_mn : lo_mn;
-      mx = (hi_mx > lo_mx) ? hi_mx : lo_mx;
+      mn = fminf(mn, __shfl_xor(mn, mask));
+      mx = fmaxf(mx, __shfl_xor(mx, mask));
     }
 
     uint16_t scale_bits;
@@ -120,17 +125,20 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
       } else if (zero_point_fp > 15.0f) {
         zp = 15;
       } else {
-        zp = static_cast<uint32_t>(roundf(zero_point_fp));
+        zp = round_0_to_15(zero_point_fp);
       }
       scale_bits = float_to_half_bits(scale_f);
     } else {
       // reference: range2scale, f16_quant_sm80.cuh:124-135
       const float m = fabsf(mx) > fabsf(mn) ? mx : mn;
       scale_bits = float_to_half_bits(__fdiv_rn(m, -8.0f));
-      // (+-0) / -8 is a zero of the opposite sign (an all-zero block gives the scale -0.0).  The
-      // compiler may evaluate the division as fma(m, -0.125, +0), which loses that sign, so the
-      // zero case takes its sign from the bits of m.
-      if (m == 0.0f) scale_bits = static_cast<uint16_t>((~__float_as_uint(m) >> 16) & 0x8000u);
+      // (+-0) / -8 is a zero of the opposite sign (an all-zero block of +0 gives the scale -0.0): the
+      // zero case takes its sign from the bits of the block's first weight, which is the value the
+      // reference's scan ends with.
+      if (m == 0.0f) {
+        const uint32_t first = __shfl(words[0], lane & ~(kLanesPerBlock - 1));  // block's first weight, fp16 bits
+        scale_bits = static_cast<uint16_t>(~first & 0x8000u);
+      }
       zp = 8;
     }
 
@@ -141,9 +149,10 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
     uint32_t word = 0;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-      float r = roundf(__fmaf_rn(v[t], reciprocal_scale, zp_f));
-      r = fmaxf(0.0f, fminf(15.0f, r));
-      word |= static_cast<uint32_t>(r) << nibble_shift(t);
+      // clamping before rounding gives the same nibble as the reference's round-then-clamp (both
+      // are monotonic)
+      const float r = __builtin_amdgcn_fmed3f(__fmaf_rn(v[t], reciprocal_scale, zp_f), 0.0f, 15.0f);
+      word |= round_0_to_15(r) << nibble_shift(t);
     }
 
     w_lds[kl >> 5][nl][(kl >> 3) & 3] = word;
