@@ -3,7 +3,7 @@
 // The work is a stream over the packed weights (K*N/2 bytes plus scales and zero-points) that has to
 // run at HBM speed; everything else is arranged so that the stream is requested as early and as
 // deeply as possible and nothing serialises behind it:
-//   - a workgroup of four waves owns 16, 32 or 48 output columns and the whole K range; the waves split K in
+//   - a workgroup of four or eight waves owns 16, 32 or 48 output columns and the whole K range; the waves split K in
 //     128-deep slices, so every wave load is one 16-byte unit per lane: 16 columns x 4 consecutive
 //     k-units = four contiguous 256-byte runs of the packed layout;
 //   - a wave keeps the weight units, scales and zero-points of kDepth slices in flight and refills a
@@ -15,7 +15,7 @@
 //   - a lane multiplies its (column, 32 k) of weights with the matching 32 k of up to 16 activation
 //     rows through v_mfma_f32_16x16x32_f16 (weights as the row operand: a lane ends up with 4
 //     consecutive output columns of one activation row, one 8-byte store);
-//   - the four partial tiles are summed through LDS by wave 0: no atomics, no scratch buffer.
+//   - the waves' partial tiles are summed through LDS by wave 0: no atomics, no scratch buffer.
 // Dequantization happens in registers (blkq4_dequant.h); accumulation is fp32.
 
 #include <hip/hip_runtime.h>
@@ -29,8 +29,6 @@ namespace {
 
 using namespace blkq4;
 
-constexpr int kThreads = 256;
-constexpr int kWaves = 4;
 
 template <int BS, int NT>
 struct Slot {
@@ -41,10 +39,10 @@ struct Slot {
   uint4 a[4];  // 32 k of this lane's activation row
 };
 
-// DEPTH: k slices (128 deep) a wave keeps in flight.  NT: 16-column tiles per wave that share one
+// kWaves: waves of the workgroup, which split K.  DEPTH: k slices (128 deep) a wave keeps in flight.  NT: 16-column tiles per wave that share one
 // activation operand.
-template <int BS, bool HAS_ZP, int DEPTH, int NT>
-__global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(const uint16_t* __restrict__ A,
+template <int BS, bool HAS_ZP, int DEPTH, int NT, int kWaves>
+__global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t* __restrict__ A,
                                                                const uint4* __restrict__ W,
                                                                const uint16_t* __restrict__ S,
                                                                const uint8_t* __restrict__ Z,
@@ -75,7 +73,7 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(const uint16_t* _
 
   const int units = K >> 5;             // 32-deep units
   const int slices = (units + 3) >> 2;  // 128-deep slices (the last one may be half full)
-  const int my_slices = (slices - wave + kWaves - 1) / kWaves;  // slices wave, wave+4, ...
+  const int my_slices = (slices - wave + kWaves - 1) / kWaves;  // slices wave, wave + kWaves, ...
 
   const int wrap_mask = (1 << (31 - __builtin_clz(units))) - 1;  // any index & wrap_mask is < units
 
@@ -191,23 +189,29 @@ void choose_shape(int m, int n, int* nt, int* depth) {
 
 template <int BS>
 int launch_skinny(const blkq4_gemm_args* a) {
-  const dim3 block(kThreads);
   hipStream_t stream = static_cast<hipStream_t>(a->stream);
   const auto* A = static_cast<const uint16_t*>(a->a);
   const auto* W = static_cast<const uint4*>(a->packed_w);
   const auto* S = static_cast<const uint16_t*>(a->scales);
   const auto* Z = static_cast<const uint8_t*>(a->zero_points);
   auto* C = static_cast<uint16_t*>(a->c);
-#define BLKQ4_LAUNCH(ZP_, DEPTH_, NT_)                                                                         \
-  hipLaunchKernelGGL((skinny_mfma_kernel<BS, ZP_, DEPTH_, NT_>), dim3((a->n / 16 + NT_ - 1) / NT_), block, 0, stream, A, W, \
-                     S, Z, C, a->m, a->n, a->k)
+#define BLKQ4_LAUNCH(ZP_, DEPTH_, NT_)                                                                  \
+  if (waves == 8)                                                                                       \
+    hipLaunchKernelGGL((skinny_mfma_kernel<BS, ZP_, (DEPTH_ > 4 ? 4 : DEPTH_), NT_, 8>),                \
+                       dim3((a->n / 16 + NT_ - 1) / NT_), dim3(512), 0, stream, A, W, S, Z, C, a->m, a->n, a->k); \
+  else                                                                                                  \
+    hipLaunchKernelGGL((skinny_mfma_kernel<BS, ZP_, DEPTH_, NT_, 4>), dim3((a->n / 16 + NT_ - 1) / NT_), \
+                       dim3(256), 0, stream, A, W, S, Z, C, a->m, a->n, a->k)
   int nt, depth;
   choose_shape(a->m, a->n, &nt, &depth);
+  // eight waves split K when there is enough of it: each wave has less to convert after its last
+  // load has arrived, and more of that work overlaps the loads of the other waves
+  const int waves = (a->k >= 1024) ? 8 : 4;
 #define BLKQ4_LAUNCH_ZP(ZP_)                   \
-  if (nt == 1 && depth == 8) BLKQ4_LAUNCH(ZP_, 8, 1); \
-  else if (nt == 1) BLKQ4_LAUNCH(ZP_, 4, 1);   \
-  else if (nt == 2) BLKQ4_LAUNCH(ZP_, 4, 2);   \
-  else BLKQ4_LAUNCH(ZP_, 4, 3)
+  if (nt == 1 && depth == 8) { BLKQ4_LAUNCH(ZP_, 8, 1); } \
+  else if (nt == 1) { BLKQ4_LAUNCH(ZP_, 4, 1); }   \
+  else if (nt == 2) { BLKQ4_LAUNCH(ZP_, 4, 2); }   \
+  else { BLKQ4_LAUNCH(ZP_, 4, 3); }
   if (Z) { BLKQ4_LAUNCH_ZP(true); } else { BLKQ4_LAUNCH_ZP(false); }
 #undef BLKQ4_LAUNCH_ZP
 #undef BLKQ4_LAUNCH
