@@ -129,10 +129,6 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_sm80(int block_size, bool column_wi
                        " is smaller than the number of rows: " + std::to_string(rows));
     return -1;
   }
-  if (!column_wise_blocking) {
-    set_error(err, kRowWiseMessage);
-    return -1;
-  }
   if (weights == nullptr || quant_weights == nullptr || quant_scales == nullptr) {
     set_error(err, "Null tensor pointer");
     return -1;
@@ -140,6 +136,7 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_sm80(int block_size, bool column_wi
 
   blkq4_prepack_args args{};
   args.block_size = block_size;
+  args.column_wise = column_wise_blocking ? 1 : 0;
   args.rows = rows;
   args.columns = columns;
   args.ld = leadingDimension;

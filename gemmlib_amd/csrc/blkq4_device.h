@@ -16,6 +16,12 @@
  *       fully coalesced 512 B / 1 KiB request.
  *   scales          fp16 [K/bs][N] row-major   (identical to the reference's packed scales)
  *   zero-points     uint8 [K/bs][N] row-major  (identical to the reference's packed offsets)
+ *
+ * With blocks along N (column_wise = 0: one k, bs consecutive columns) the packed weights are the
+ * same and the meta data keep the reference's packed order for that blocking: column-major
+ * [K][N/bs] (element (k, g) in the 16-row group starting at g*K + (k & ~15)), and inside a group of
+ * 16 rows the scales of rows (2t, 2t+1, 2t+8, 2t+9) and the zero-points of rows (2t, 2t+8, 2t+1,
+ * 2t+9) sit at positions 4t .. 4t+3, t = 0..3.
  */
 
 #pragma once
@@ -29,6 +35,7 @@ extern "C" {
 
 typedef struct {
   int block_size;      /* 16, 32 or 64 */
+  int column_wise;     /* 1: blocks of bs x 1 (along K); 0: blocks of 1 x bs (along N) */
   int rows;            /* K, multiple of 64 */
   int columns;         /* N, multiple of 32 */
   int ld;              /* leading dimension of the fp16 source, >= rows */
@@ -41,6 +48,7 @@ typedef struct {
 
 typedef struct {
   int block_size;
+  int column_wise;          /* as in blkq4_prepack_args */
   int m, n, k;
   const void* a;            /* fp16 [m][k] */
   const void* packed_w;     /* uint8[K/32][N][16] */

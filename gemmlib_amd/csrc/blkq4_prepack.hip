@@ -204,6 +204,159 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
 }
 
 // ------------------------------------------------------------------------------------------------
+// Row-wise blocking: a quantization block is one k and BS consecutive columns, so every k of a lane's
+// eight has its own scale and zero-point (reference: the [1, bs] block shape of
+// src/mickey/blk_q4/f16_quant_sm80.cuh:206-212, 225-315).  Same tile, same packed weight layout and
+// the same arithmetic as above; only the reduction runs across columns.  A wave covers 64 k of all
+// 64 columns of the tile: lane = (column & 7) * 8 + (k / 8), eight passes of 8 columns, so a block
+// is BS/8 passes times 8 lanes.
+//
+// Scales and zero-points leave in the reference's packed order for this blocking
+// (f16_quant_sm80.cuh:506-512, 528-539): column-major [K][N/BS], and inside every group of 16
+// rows scale rows (2t, 2t+1, 2t+8, 2t+9) and zero-point rows (2t, 2t+8, 2t+1, 2t+9) sit at
+// positions 4t .. 4t+3.
+// ------------------------------------------------------------------------------------------------
+template <int BS, bool HAS_ZP, bool ALIGNED>
+__global__ __launch_bounds__(kThreads) void prepack_rowwise_kernel(const uint16_t* __restrict__ src, int K,
+                                                                   int N, int ld,
+                                                                   uint4* __restrict__ packed_w,
+                                                                   uint16_t* __restrict__ scales,
+                                                                   uint8_t* __restrict__ zps, unsigned k_tiles) {
+  constexpr int kPasses = BS / 8;            // passes of 8 columns that make up one block
+  constexpr int kGroups = kTileN / BS;       // blocks along N in one tile
+  __shared__ uint32_t w_lds[kTileK / 32][kTileN][4];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int c8 = lane >> 3;  // column inside a pass
+  const int kq = lane & 7;   // which 8 k of the wave's 64
+  const int k0 = static_cast<int>(blockIdx.x % k_tiles) * kTileK;
+  const int n0 = static_cast<int>(blockIdx.x / k_tiles) * kTileN;
+  const int kl = wave * 64 + kq * 8;  // this lane's first k inside the tile
+  const bool k_ok = (k0 + kl) < K;    // K is a multiple of 64: a wave's 64 k are all in or all out
+
+  uint4 raw[8];
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int n = n0 + it * 8 + c8;
+    raw[it] = make_uint4(0, 0, 0, 0);
+    if (k_ok && n < N) {  // N is a multiple of BS: a block is all in or all out
+      const uint16_t* p = src + static_cast<size_t>(n) * ld + (k0 + kl);
+      if constexpr (ALIGNED) {
+        raw[it] = *reinterpret_cast<const uint4*>(p);
+      } else {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = static_cast<uint32_t>(p[2 * i]) | (static_cast<uint32_t>(p[2 * i + 1]) << 16);
+        raw[it] = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+    }
+  }
+#define BLKQ4_VALUE(it_, t_) \
+  half_bits_to_float((((t_) >> 1) == 0 ? raw[it_].x : ((t_) >> 1) == 1 ? raw[it_].y : ((t_) >> 1) == 2 ? raw[it_].z : raw[it_].w) >> (16 * ((t_) & 1)) & 0xffffu)
+
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g) {
+    float rs[8], zf[8];
+    uint32_t sbits[8], zq[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      // range of the block of k = k0 + kl + t: the passes of this group, then the 8 column lanes
+      float mn = BLKQ4_VALUE(g * kPasses, t), mx = mn;
+#pragma unroll
+      for (int q = 1; q < kPasses; ++q) {
+        const float v = BLKQ4_VALUE(g * kPasses + q, t);
+        mn = fminf(mn, v);
+        mx = fmaxf(mx, v);
+      }
+#pragma unroll
+      for (int mask = 8; mask < 64; mask <<= 1) {
+        mn = fminf(mn, __shfl_xor(mn, mask));
+        mx = fmaxf(mx, __shfl_xor(mx, mask));
+      }
+      uint16_t scale_bits;
+      uint32_t zp;
+      if constexpr (HAS_ZP) {
+        const float rmn = fminf(mn, 0.0f);
+        const float rmx = fmaxf(mx, 0.0f);
+        const float scale_f = div_by_15(__fsub_rn(rmx, rmn));
+        float zero_point_fp = rmn;
+        if (scale_f != 0.0f) zero_point_fp = __fsub_rn(0.0f, __fdiv_rn(rmn, scale_f));
+        if (zero_point_fp < 0.0f) {
+          zp = 0;
+        } else if (zero_point_fp > 15.0f) {
+          zp = 15;
+        } else {
+          zp = round_0_to_15(zero_point_fp);
+        }
+        scale_bits = float_to_half_bits(scale_f);
+      } else {
+        const float m = fabsf(mx) > fabsf(mn) ? mx : mn;
+        scale_bits = float_to_half_bits(__fdiv_rn(m, -8.0f));
+        if (m == 0.0f) {
+          // all-zero block: the sign comes from the block's first weight (its first column, this k)
+          const uint32_t w0 = ((t >> 1) == 0 ? raw[g * kPasses].x : (t >> 1) == 1 ? raw[g * kPasses].y
+                               : (t >> 1) == 2 ? raw[g * kPasses].z : raw[g * kPasses].w) >> (16 * (t & 1));
+          const uint32_t first = __shfl(w0, kq);
+          scale_bits = static_cast<uint16_t>(~first & 0x8000u);
+        }
+        zp = 8;
+      }
+      const float scale = half_bits_to_float(scale_bits);
+      rs[t] = (scale != 0.0f) ? __fdiv_rn(1.0f, scale) : 0.0f;
+      zf[t] = static_cast<float>(zp);
+      sbits[t] = scale_bits;
+      zq[t] = zp;
+    }
+#pragma unroll
+    for (int q = 0; q < kPasses; ++q) {
+      const int it = g * kPasses + q;
+      uint32_t word = 0;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const float r = __builtin_amdgcn_fmed3f(__fmaf_rn(BLKQ4_VALUE(it, t), rs[t], zf[t]), 0.0f, 15.0f);
+        word |= round_0_to_15(r) << nibble_shift(t);
+      }
+      w_lds[kl >> 5][it * 8 + c8][(kl >> 3) & 3] = word;
+    }
+    // meta data of the group: one lane per 8 rows writes them
+    const int n_first = n0 + g * BS;
+    if (c8 == 0 && k_ok && n_first < N) {
+      const int row16 = (k0 + kl) & ~15;   // first row of the 16-row group
+      const int upper = ((k0 + kl) >> 3) & 1;  // this lane holds rows 8..15 of the group
+      const size_t base = static_cast<size_t>(n_first / BS) * K + row16;
+#pragma unroll
+      for (int tp = 0; tp < 4; ++tp) {
+        // rows (2tp, 2tp+1) of this lane's eight
+        const uint32_t pair = sbits[2 * tp] | (sbits[2 * tp + 1] << 16);
+        *reinterpret_cast<uint32_t*>(scales + base + 4 * tp + 2 * upper) = pair;
+        if constexpr (HAS_ZP) {
+          zps[base + 4 * tp + upper] = static_cast<uint8_t>(zq[2 * tp]);
+          zps[base + 4 * tp + upper + 2] = static_cast<uint8_t>(zq[2 * tp + 1]);
+        }
+      }
+    }
+  }
+#undef BLKQ4_VALUE
+  __syncthreads();
+
+  // packed weights: one 16-byte unit per thread and pass, 1 KiB contiguous per wave
+#pragma unroll
+  for (int r = 0; r < (kTileK / 32) * kTileN / kThreads; ++r) {
+    const int u = tid + r * kThreads;
+    const int ksl = u / kTileN;
+    const int nl = u % kTileN;
+    const int k = k0 + ksl * 32;
+    const int n = n0 + nl;
+    if (k < K && n < N) {
+      const uint4 val = *reinterpret_cast<const uint4*>(&w_lds[ksl][nl][0]);
+      packed_w[static_cast<size_t>(k >> 5) * N + n] = val;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Layout conversion between the packed layout above and the reference's sm80 layout
 // (reference: src/mickey/blk_q4/f16_quant_sm80.cuh:362-417): uint8[K, N/2] column-major, where for
 // each 16x16 weight tile at (k0, n0), row in 0..3, col in 0..7, s in 0..3 the byte at
@@ -263,7 +416,31 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__
 }
 
 template <int BS>
+int launch_prepack_rowwise(const blkq4_prepack_args* a) {
+  const unsigned k_tiles = (a->rows + kTileK - 1) / kTileK;
+  const dim3 grid(k_tiles * static_cast<unsigned>((a->columns + kTileN - 1) / kTileN));
+  const dim3 block(kThreads);
+  hipStream_t stream = static_cast<hipStream_t>(a->stream);
+  const auto* src = static_cast<const uint16_t*>(a->src);
+  auto* pw = static_cast<uint4*>(a->packed_w);
+  auto* sc = static_cast<uint16_t*>(a->scales);
+  auto* zp = static_cast<uint8_t*>(a->zero_points);
+  const bool aligned = (reinterpret_cast<uintptr_t>(a->src) & 15u) == 0 && (a->ld % 8) == 0;
+#define BLKQ4_LAUNCH(ZP_, AL_)                                                                                   \
+  hipLaunchKernelGGL((prepack_rowwise_kernel<BS, ZP_, AL_>), grid, block, 0, stream, src, a->rows, a->columns, \
+                     a->ld, pw, sc, zp, k_tiles)
+  if (zp) {
+    if (aligned) BLKQ4_LAUNCH(true, true); else BLKQ4_LAUNCH(true, false);
+  } else {
+    if (aligned) BLKQ4_LAUNCH(false, true); else BLKQ4_LAUNCH(false, false);
+  }
+#undef BLKQ4_LAUNCH
+  return static_cast<int>(hipGetLastError());
+}
+
+template <int BS>
 int launch_prepack(const blkq4_prepack_args* a) {
+  if (!a->column_wise) return launch_prepack_rowwise<BS>(a);
   const unsigned k_tiles = (a->rows + kTileK - 1) / kTileK;
   const dim3 grid(k_tiles * static_cast<unsigned>((a->columns + kTileN - 1) / kTileN));
   const dim3 block(kThreads);
@@ -294,6 +471,10 @@ int launch_prepack(const blkq4_prepack_args* a) {
 
 extern "C" int blkq4_dev_prepack(const blkq4_prepack_args* a) {
   if ((reinterpret_cast<uintptr_t>(a->packed_w) & 15u) != 0) return static_cast<int>(hipErrorInvalidValue);
+  // row-wise blocking: scale pairs are stored as 32-bit words; a block may not straddle the tile edge
+  if (!a->column_wise && ((reinterpret_cast<uintptr_t>(a->scales) & 3u) != 0 || (a->columns % a->block_size) != 0)) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
   switch (a->block_size) {
     case 16: return launch_prepack<16>(a);
     case 32: return launch_prepack<32>(a);

@@ -133,7 +133,7 @@ def _quant(capi, bs=32, col=True, rows=64, cols=32, ld=None, src=None, qw=None, 
     (dict(qz=_buf(63)), "Unexpected offset tensor size: 63 expected: 64"),
     (dict(src=_buf(64 * 32 * 2 - 2)), "Unexpected weight tensor size: 2047 expected: 2048"),
     (dict(ld=80, src=_buf(64 * 32 * 2)), "Unexpected weight tensor size: 2048 expected: 2560"),
-    (dict(col=False, qs=_buf(64 * 2)), "Row-wise blocking (column_wise_blocking = false) is not implemented by this library"),
+    (dict(col=False, qs=_buf(60 * 2)), "Unexpected scale tensor size: 60 expected: 64"),   # row-wise meta is [K, N/bs]
 ])
 def test_quant_validation_messages(capi, kwargs, message):
     rc, text = _quant(capi, **kwargs)

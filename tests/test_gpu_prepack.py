@@ -26,11 +26,11 @@ def digest(a) -> str:
     return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()[:16]
 
 
-def check_against_oracle(oracle, capi, device, bs, weights_nk, has_offsets, w_dev=None):
+def check_against_oracle(oracle, capi, device, bs, weights_nk, has_offsets, w_dev=None, column_wise=True):
     n, k = weights_nk.shape
-    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, weights_nk, has_offsets, w_dev)
-    canon, s, z = oracle.quantize(bs, True, weights_nk, has_offsets)
-    ps, pz = oracle.prepack_meta_sm80(bs, True, k, n, s, z)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, weights_nk, has_offsets, w_dev, column_wise)
+    canon, s, z = oracle.quantize(bs, column_wise, weights_nk, has_offsets)
+    ps, pz = oracle.prepack_meta_sm80(bs, column_wise, k, n, s, z)
     got_s = to_np(q_s)
     assert np.array_equal(got_s.view(np.uint16), ps.view(np.uint16)), "scales differ"
     if has_offsets:
@@ -65,16 +65,37 @@ def test_reference_known_answers(oracle, capi, device, rows, columns, has_offset
 
 
 def test_reference_known_answer_digests(oracle, capi, device):
+    """both blockings (reference: test/blkq4_fp16_quant_sm80_test.cu:313-347)."""
     with open(os.path.join(GOLDEN, "kat_digests_independent.json")) as f:
         table = json.load(f)
     for case in table["cases"]:
-        if not case["column_wise"]:
-            continue
-        kat = oracle.kat_generate(32, True, case["rows"], case["columns"], True)
-        sm80, s, z, _ = check_against_oracle(oracle, capi, device, 32, kat["weights"], True)
+        col = bool(case["column_wise"])
+        kat = oracle.kat_generate(32, col, case["rows"], case["columns"], True)
+        sm80, s, z, _ = check_against_oracle(oracle, capi, device, 32, kat["weights"], True, column_wise=col)
         assert digest(sm80) == case["packedW"]
         assert digest(s.view(np.uint16)) == case["packedS"]
         assert digest(z) == case["packedZ"]
+
+
+@pytest.mark.parametrize("rows,columns", KAT_SHAPES)
+@pytest.mark.parametrize("has_offsets", [True, False])
+def test_reference_known_answers_rowwise(oracle, capi, device, rows, columns, has_offsets):
+    """blocks of 1 x 32 along N (reference: test/blkq4_fp16_quant_sm80_test.cu:313-334)."""
+    kat = oracle.kat_generate(32, False, rows, columns, has_offsets)
+    _, _, _, canon = check_against_oracle(oracle, capi, device, 32, kat["weights"], has_offsets, column_wise=False)
+    assert np.array_equal(canon, kat["canon_w"])
+
+
+@pytest.mark.parametrize("bs", [16, 32, 64])
+@pytest.mark.parametrize("has_offsets", [True, False])
+@pytest.mark.parametrize("rows,columns", [(64, 64), (192, 192), (320, 448), (1024, 1024)])
+def test_gaussian_rowwise(oracle, capi, device, bs, has_offsets, rows, columns):
+    rng = np.random.default_rng(bs * 104729 + rows * 31 + columns + has_offsets)
+    w = (rng.standard_normal((columns, rows)) * 0.02).astype(np.float16)
+    w[0, :] = 0.0                    # all-zero blocks, and blocks whose first weight is -0
+    w[:, 3] = -0.0
+    w[5, 7] = 0.0
+    check_against_oracle(oracle, capi, device, bs, w, has_offsets, column_wise=False)
 
 
 @pytest.mark.parametrize("bs", [16, 32, 64])
