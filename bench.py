@@ -28,21 +28,48 @@ PEAK_MFMA_TFLOPS = 2500.0   # fp16 dense MFMA, MI355X published
 PEAK_HBM_GBPS = 8000.0      # HBM3E, MI355X published
 INFINITY_CACHE_BYTES = 256 << 20
 
-# name: (M, K, N, block_size, has_offsets, bound)
+# name: (M, K, N, block_size, has_offsets, bound); blocks run along K except where COLUMN_WISE says otherwise
 CONFIGS = {
     "C1": (64, 1024, 1024, 32, True, "mfma"),
     "C2": (1, 4096, 4096, 64, False, "hbm"),
     "C3": (16, 4096, 11008, 32, True, "hbm"),
     "C4": (2048, 4096, 4096, 64, True, "mfma"),
     "C5": (4096, 8192, 28672, 16, True, "mfma"),
+    "C4r": (2048, 4096, 4096, 64, True, "mfma"),
 }
+COLUMN_WISE = {"C4r": False}
 DESCRIPTION = {
     "C1": "C1 CPU-runnable case M=64 K=1024 N=1024 bs32 asym",
     "C2": "C2 decode GEMV M=1 K=4096 N=4096 bs64 sym",
     "C3": "C3 skinny GEMM M=16 K=4096 N=11008 bs32 asym",
     "C4": "C4 prefill GEMM M=2048 K=4096 N=4096 bs64 asym",
     "C5": "C5 large-layer GEMM M=4096 K=8192 N=28672 bs16 asym",
+    "C4r": "C4 shape with blocks along N (column_wise_blocking=false) M=2048 K=4096 N=4096 bs64 asym",
 }
+
+
+# HBM-side traffic per launch, measured with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (two runs of
+# this script, KiB per dispatch, mean over the dispatches of the kernel) and scaled by what the same counter
+# reads for the runtime's device-to-device copy of a 128 MiB buffer in the same run (FETCH_SIZE reads
+# 65 557 KiB for 131 072 KiB fetched: factor 2.0; WRITE_SIZE reads 131 072 KiB: factor 1.0).  The counters
+# sit between L2 and the memory fabric, so reads served by the Infinity Cache are included.  A script cannot
+# read these counters for itself; the figures are refreshed when a kernel changes.
+COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65557.0, "WRITE_SIZE": 1.0}
+COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
+    "C4": (44090.3, 16384.0),
+    "C2": (5191.1, 8.0),
+    "C3": (16652.1, 344.0),
+    "C5": (860293.0, 229422.0),
+    "C5_prepack": (229442.0, 158496.0),
+    "C4r": (51758.9, 30282.2),
+}
+
+
+def traffic_bytes(name):
+    if name not in COUNTER_KIB:
+        return None
+    f, w = COUNTER_KIB[name]
+    return int(round((f * COUNTER_SCALE["FETCH_SIZE"] + w * COUNTER_SCALE["WRITE_SIZE"]) * 1024))
 
 
 def algorithmic(m, k, n, bs, has_offsets):
@@ -100,9 +127,10 @@ def timed_region(torch, launches, steps, warmup):
 
 def make_problem(torch, capi, name, device, copies):
     m, k, n, bs, has_offsets, _ = CONFIGS[name]
+    col = COLUMN_WISE.get(name, True)
     g = torch.Generator(device="cpu").manual_seed(1234 + list(CONFIGS).index(name))
     a = torch.randn(m, k, generator=g, dtype=torch.float32).to(torch.float16).to(device)
-    w_elems, meta_elems = capi.quant_size(bs, True, k, n)
+    w_elems, meta_elems = capi.quant_size(bs, col, k, n)
     sets = []
     w_host = None
     for c in range(copies):
@@ -111,7 +139,7 @@ def make_problem(torch, capi, name, device, copies):
         q_w = torch.empty(w_elems, dtype=torch.uint8, device=device)
         q_s = torch.empty(meta_elems, dtype=torch.float16, device=device)
         q_zp = torch.empty(meta_elems, dtype=torch.uint8, device=device) if has_offsets else None
-        capi.quant(bs, True, w, q_w, q_s, q_zp)
+        capi.quant(bs, col, w, q_w, q_s, q_zp)
         sets.append((q_w, q_s, q_zp))
         del w
     torch.cuda.synchronize()
@@ -127,10 +155,11 @@ def bench_gemm(torch, capi, name, device, steps, warmup):
         per_set = nbytes - 2 * m * k - 2 * m * n
         copies = INFINITY_CACHE_BYTES // per_set + 2
     a, sets, out, w_host = make_problem(torch, capi, name, device, copies)
+    col = COLUMN_WISE.get(name, True)
 
     def mk(s):
         q_w, q_s, q_zp = s
-        return lambda: capi.gemm(bs, True, m, n, k, a, q_w, q_s, q_zp, out)
+        return lambda: capi.gemm(bs, col, m, n, k, a, q_w, q_s, q_zp, out)
 
     launches = [mk(s) for s in sets]
     wall, evt, mode = timed_region(torch, launches, steps, warmup)
@@ -148,7 +177,7 @@ def bench_gemm(torch, capi, name, device, steps, warmup):
         "timing": mode, "weight_sets": copies, "flops": flops, "bytes": nbytes,
         "tflops": round(flops / per_call_evt / 1e12, 3), "gbps": round(nbytes / per_call_evt / 1e9, 3),
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": None},
+                     "frac": round(achieved / peak, 4), "traffic": traffic_bytes(name)},
     }
     return res, (a, sets, out, w_host)
 
@@ -172,7 +201,7 @@ def bench_prepack(torch, capi, device, steps, warmup):
         "unit": "GB/s", "ms_per_step": round(wall / steps * 1e3, 6), "kernel_us": round(per * 1e6, 3), "timing": mode,
         "bytes": nbytes, "gbps": round(ach, 3),
         "roofline": {"bound": "hbm", "achieved": round(ach, 3), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                     "frac": round(ach / PEAK_HBM_GBPS, 4), "traffic": None},
+                     "frac": round(ach / PEAK_HBM_GBPS, 4), "traffic": traffic_bytes("C5_prepack")},
     }
 
 
@@ -186,6 +215,8 @@ def bench_copy(torch, capi, device, steps, warmup):
     dst = torch.empty_like(src)
     launches = [lambda: capi.repack(True, rows, cols, src, dst)]
     steps = max(10, steps // 10)
+    for _ in range(steps):  # the runtime's own device-to-device copy of the same buffer, as a second reference
+        dst.copy_(src)
     wall, evt, mode = timed_region(torch, launches, steps, max(2, warmup // 10))
     per = evt / steps
     ach = 2 * nbytes / per / 1e9
@@ -233,7 +264,7 @@ def main(argv=None) -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack")
+    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args(argv)
     if args.gpus != 1:

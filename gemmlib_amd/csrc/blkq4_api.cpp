@@ -23,9 +23,6 @@ inline bool supported_block_size(int bs) { return bs == 16 || bs == 32 || bs == 
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-constexpr const char* kRowWiseMessage =
-    "Row-wise blocking (column_wise_blocking = false) is not implemented by this library";
-
 // reference: src/blkq4_f16_gemm_sm80.cu:155-203 (blkq4_quant_size_sm80_T)
 int quant_size(int block_size, bool column_wise, int rows, int columns, int64_t& w_size,
                int64_t& meta_size, std::string* err) {
@@ -214,8 +211,9 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
     set_error(err, "Kernel execution failed: Error Misaligned Operand");
     return -1;
   }
-  if (!column_wise_blocking) {
-    set_error(err, kRowWiseMessage);
+  // blocks along N: the kernel fetches scales and zero-points 16 bytes at a time
+  if (!column_wise_blocking && (!aligned16(scales_ptr) || (has_offsets && !aligned16(offsets_ptr)))) {
+    set_error(err, "Kernel execution failed: Error Misaligned Operand");
     return -1;
   }
   if (act_ptr == nullptr || weights_ptr == nullptr || scales_ptr == nullptr || output_ptr == nullptr) {
@@ -225,6 +223,7 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
 
   blkq4_gemm_args args{};
   args.block_size = block_size;
+  args.column_wise = column_wise_blocking ? 1 : 0;
   args.m = m;
   args.n = n;
   args.k = k;
@@ -235,7 +234,9 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
   args.c = output_ptr;
   args.stream = stream;
   // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
-  const int code = (m > 16) ? blkq4_dev_gemm(&args) : blkq4_dev_skinny(&args);
+  const int code = !column_wise_blocking ? blkq4_dev_gemm_rowwise(&args)
+                   : (m > 16)            ? blkq4_dev_gemm(&args)
+                                         : blkq4_dev_skinny(&args);
   if (code) return device_failure(code, err);
   return 0;
 }

@@ -52,8 +52,8 @@ typedef struct {
   int m, n, k;
   const void* a;            /* fp16 [m][k] */
   const void* packed_w;     /* uint8[K/32][N][16] */
-  const void* scales;       /* fp16 [K/bs][N] */
-  const void* zero_points;  /* uint8 [K/bs][N] or NULL */
+  const void* scales;       /* fp16 [K/bs][N]; column_wise = 0: packed [K][N/bs] order described above */
+  const void* zero_points;  /* uint8, same shape and order as the scales, or NULL */
   void* c;                  /* fp16 [m][n] */
   void* stream;
 } blkq4_gemm_args;
@@ -69,6 +69,7 @@ typedef struct {
 int blkq4_dev_prepack(const blkq4_prepack_args* args);
 int blkq4_dev_gemm(const blkq4_gemm_args* args);   /* m > 16: MFMA tile kernel */
 int blkq4_dev_skinny(const blkq4_gemm_args* args); /* 1 <= m <= 16 */
+int blkq4_dev_gemm_rowwise(const blkq4_gemm_args* args); /* column_wise = 0, every m */
 int blkq4_dev_repack(const blkq4_repack_args* args);
 const char* blkq4_dev_error_string(int code);
 

@@ -99,7 +99,10 @@ def _gemm(capi, bs=32, col=True, m=4, n=64, k=64, a=None, w=None, s=None, z=None
      "Kernel execution failed: Error Invalid Problem"),
     (dict(a=_buf(512, address=0x1002)), "Kernel execution failed: Error Misaligned Operand"),
     (dict(c=_buf(512, address=0x1008)), "Kernel execution failed: Error Misaligned Operand"),
-    (dict(col=False, s=_buf(64 * 2 * 2)), "Row-wise blocking (column_wise_blocking = false) is not implemented by this library"),
+    # blocks along N: the scales are fetched 16 bytes at a time; n must be a multiple of the block size
+    (dict(col=False, s=_buf(64 * 2 * 2, address=0x1004)), "Kernel execution failed: Error Misaligned Operand"),
+    (dict(col=False, bs=64, n=96, w=_buf(64 * 96 // 2), s=_buf(64 * 1 * 2), c=_buf(4 * 96 * 2)),
+     "Kernel execution failed: Error Invalid Problem"),
 ])
 def test_gemm_validation_messages(capi, kwargs, message):
     with pytest.raises(capi.Blkq4Error) as e:
