@@ -9,9 +9,11 @@
 //   - a wave keeps the weight units, scales and zero-points of kDepth slices in flight and refills a
 //     slot as soon as it has consumed it (out-of-range slices wrap around to valid units and are
 //     multiplied by a zero scale, so the loop has no divergent loads);
-//   - the lanes that carry an activation row load their 64 bytes per slice straight from global
-//     memory (L2 resident) into the same ring, so every request of a slice is issued together and
-//     the compiler's in-order vmcnt waits let slice i be consumed while slices i+1.. are in flight;
+//   - the activation rows (at most 16 x K fp16) are copied once per workgroup into LDS by asynchronous
+//     global_load_lds copies issued before the first weight request, laid out per 32-deep unit as
+//     [unit][row][64 bytes] (16-byte chunks XOR-swizzled with bits 2..3 of the row so that a fragment
+//     read is free of bank conflicts); when they do not fit (K too large) the lanes that carry a row
+//     load their 64 bytes per slice straight from global memory (L2 resident) into the same ring;
 //   - a lane multiplies its (column, 32 k) of weights with the matching 32 k of up to 16 activation
 //     rows through v_mfma_f32_16x16x32_f16 (weights as the row operand: a lane ends up with 4
 //     consecutive output columns of one activation row, one 8-byte store);
@@ -24,32 +26,37 @@
 
 #include "blkq4_dequant.h"
 #include "blkq4_device.h"
+#include "blkq4_gemm_common.h"
 
 namespace {
 
 using namespace blkq4;
 
 
-template <int BS, int NT>
+template <int BS, int NT, bool A_LDS>
 struct Slot {
   static constexpr int kMeta = (BS == 16) ? 2 : 1;  // quantization blocks inside one 32-deep unit
   uint4 w[NT];
   uint32_t sc[NT][kMeta];
   uint32_t zp[NT][kMeta];
-  uint4 a[4];  // 32 k of this lane's activation row
+  uint4 a[A_LDS ? 1 : 4];  // 32 k of this lane's activation row (unused when the rows are in LDS)
 };
 
 // kWaves: waves of the workgroup, which split K.  DEPTH: k slices (128 deep) a wave keeps in flight.  NT: 16-column tiles per wave that share one
-// activation operand.
-template <int BS, bool HAS_ZP, int DEPTH, int NT, int kWaves>
+// activation operand.  A_LDS: the activation rows are staged in LDS (rows_log2 = log2 of the number of rows
+// kept there, a power of two >= M); the dynamic LDS size is red_bytes + (K * 2 << rows_log2).
+template <int BS, bool HAS_ZP, int DEPTH, int NT, int kWaves, bool A_LDS>
 __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t* __restrict__ A,
                                                                const uint4* __restrict__ W,
                                                                const uint16_t* __restrict__ S,
                                                                const uint8_t* __restrict__ Z,
                                                                uint16_t* __restrict__ C, int M, int N,
-                                                               int K) {
-  constexpr int kMeta = Slot<BS, NT>::kMeta;
-  __shared__ float red[kWaves * NT * 64 * 4];
+                                                               int K, int rows_log2) {
+  constexpr int kMeta = Slot<BS, NT, A_LDS>::kMeta;
+  constexpr int kRedFloats = kWaves * NT * 64 * 4;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  float* red = reinterpret_cast<float*>(smem);
+  const uint8_t* a_lds = smem + kRedFloats * 4;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -80,7 +87,28 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   float4_t acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
-  Slot<BS, NT> slot[DEPTH];
+  Slot<BS, NT, A_LDS> slot[DEPTH];
+
+  // Rows to LDS: copy q fills LDS bytes [1024 q, 1024 q + 1024) of the [unit][row][64 B] layout, lane l
+  // the 16 bytes at 16 l.  They are requested before anything else, so every later wait covers them.
+  uint32_t a_rd = 0;  // LDS byte offset of this lane's row inside a unit, chunk 0
+  uint32_t a_swz = 0;
+  if (A_LDS) {
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+                              (__attribute__((address_space(3))) uint8_t*)(smem))) + kRedFloats * 4;
+    const int rows = 1 << rows_log2;
+    const int copies = ((K << rows_log2) + 511) >> 9;  // K * 2 * rows bytes in 1 KiB copies, the last one may be partial
+    for (int q = wave; q < copies; q += kWaves) {
+      const uint32_t off = q * 1024 + lane * 16;
+      const int u = min(static_cast<int>(off >> (6 + rows_log2)), units - 1);  // past the end: any valid unit
+      const int row = (off >> 6) & (rows - 1);
+      const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+      async_copy_16(lds0 + q * 1024, A, (static_cast<uint32_t>(min(row, M - 1)) * K + u * 32 + chunk * 8) * 2);
+    }
+    const int row = min(nl, rows - 1);
+    a_rd = row * 64;
+    a_swz = (row >> 2) & 3;
+  }
   // a slice past the end wraps around to valid units (so every slot always issues the same loads)
   // and gets a zero scale, which makes it contribute exactly 0
 #define BLKQ4_LOAD_SLOT(dst_, slice_)                                                          \
@@ -98,21 +126,37 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
         (dst_).zp[t][q] = HAS_ZP ? static_cast<uint32_t>(Z[mi_]) : 8u;                         \
       }                                                                                        \
     }                                                                                          \
-    const uint4* p_ = reinterpret_cast<const uint4*>(a_row + static_cast<size_t>(ksg_) * 64);  \
-    if (row_ok) {                                                                              \
-      _Pragma("unroll") for (int j = 0; j < 4; ++j)(dst_).a[j] = p_[j];                        \
+    if (!A_LDS) {                                                                              \
+      const uint4* p_ = reinterpret_cast<const uint4*>(a_row + static_cast<size_t>(ksg_) * 64);\
+      if (row_ok) {                                                                            \
+        _Pragma("unroll") for (int j = 0; j < (A_LDS ? 1 : 4); ++j)(dst_).a[j] = p_[j];        \
+      }                                                                                        \
     }                                                                                          \
   }
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) BLKQ4_LOAD_SLOT(slot[d], wave + d * kWaves);
+  if (A_LDS) {
+    // everything but the requests of the ring just issued has landed: this wave's share of the rows
+    constexpr int kRing = DEPTH * NT * (1 + kMeta * (HAS_ZP ? 2 : 1));
+    wait_vmcnt<(kRing < 63 ? kRing : 63)>();
+    __syncthreads();
+  }
 
   for (int i0 = 0; i0 < my_slices; i0 += DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       const int li = i0 + d;  // local slice index; slice = wave + 4*li
       half8_t af[4];
+      if (A_LDS) {
+        const int ks = 4 * (wave + kWaves * li) + g;
+        const int ksg = (ks < units) ? ks : (ks & wrap_mask);
+        const uint8_t* ap = a_lds + (static_cast<uint32_t>(ksg) << (6 + rows_log2)) + a_rd;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) af[j] = as_half8(slot[d].a[j]);
+        for (int j = 0; j < 4; ++j) af[j] = as_half8(*reinterpret_cast<const uint4*>(ap + ((j ^ a_swz) * 16)));
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) af[j] = as_half8(slot[d].a[j < (A_LDS ? 1 : 4) ? j : 0]);
+      }
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         DequantConsts dc[kMeta];
@@ -142,23 +186,16 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 #pragma unroll
     for (int e = 0; e < 4; ++e) red[((wave * NT + t) * 64 + lane) * 4 + e] = acc[t][e];
   __syncthreads();
-  if (wave == 0) {
+  // value v = (tile t, lane L, element e) of the partial tiles: output row L & 15, column 4 (L >> 4) + e
+  // of tile t; every thread sums a few of them over the waves
+  for (int v = tid; v < NT * 256; v += 64 * kWaves) {
+    float r = 0.f;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      float r[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        r[e] = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) r[e] += red[((w * NT + t) * 64 + lane) * 4 + e];
-      }
-      if (row_ok && blockIdx.x * NT + t < tiles) {
-        // lane (row nl, group g) holds output columns 4g .. 4g+3 of 16-column tile t
-        const uint32_t lo = float_to_half_bits(r[0]) | (static_cast<uint32_t>(float_to_half_bits(r[1])) << 16);
-        const uint32_t hi = float_to_half_bits(r[2]) | (static_cast<uint32_t>(float_to_half_bits(r[3])) << 16);
-        uint2* out = reinterpret_cast<uint2*>(C + static_cast<size_t>(nl) * N + blockIdx.x * (16 * NT) + 16 * t + 4 * g);
-        *out = make_uint2(lo, hi);
-      }
+    for (int w = 0; w < kWaves; ++w) r += red[w * (NT * 256) + v];
+    const int t = v >> 8, L = (v >> 2) & 63, e = v & 3;
+    const int row = L & 15;
+    if (row < M && blockIdx.x * NT + t < tiles) {
+      C[static_cast<size_t>(row) * N + blockIdx.x * (16 * NT) + 16 * t + 4 * (L >> 4) + e] = float_to_half_bits(r);
     }
   }
 }
@@ -167,6 +204,11 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 // evenly the workgroups fill the 256 compute units: with T column tiles per workgroup the busiest
 // unit works through ceil(workgroups / 256) * T tiles.  Wider workgroups also re-read the activation
 // rows less often, which weighs more the more rows there are.
+constexpr size_t kMaxLdsBytes = 160 * 1024;
+#ifndef BLKQ4_SKINNY_WAVES16
+#define BLKQ4_SKINNY_WAVES16 1
+#endif
+
 void choose_shape(int m, int n, int* nt, int* depth) {
   constexpr int kComputeUnits = 256;
   const int tiles = n / 16;
@@ -187,35 +229,57 @@ void choose_shape(int m, int n, int* nt, int* depth) {
   *depth = (*nt == 1 && tiles <= 2 * kComputeUnits) ? 8 : 4;
 }
 
-template <int BS>
-int launch_skinny(const blkq4_gemm_args* a) {
-  hipStream_t stream = static_cast<hipStream_t>(a->stream);
-  const auto* A = static_cast<const uint16_t*>(a->a);
-  const auto* W = static_cast<const uint4*>(a->packed_w);
-  const auto* S = static_cast<const uint16_t*>(a->scales);
-  const auto* Z = static_cast<const uint8_t*>(a->zero_points);
-  auto* C = static_cast<uint16_t*>(a->c);
-#define BLKQ4_LAUNCH(ZP_, DEPTH_, NT_)                                                                  \
-  if (waves == 8)                                                                                       \
-    hipLaunchKernelGGL((skinny_mfma_kernel<BS, ZP_, (DEPTH_ > 4 ? 4 : DEPTH_), NT_, 8>),                \
-                       dim3((a->n / 16 + NT_ - 1) / NT_), dim3(512), 0, stream, A, W, S, Z, C, a->m, a->n, a->k); \
-  else                                                                                                  \
-    hipLaunchKernelGGL((skinny_mfma_kernel<BS, ZP_, DEPTH_, NT_, 4>), dim3((a->n / 16 + NT_ - 1) / NT_), \
-                       dim3(256), 0, stream, A, W, S, Z, C, a->m, a->n, a->k)
-  int nt, depth;
-  choose_shape(a->m, a->n, &nt, &depth);
+// One kernel instantiation: raises its dynamic-LDS limit once, then launches.
+template <int BS, bool HAS_ZP, int DEPTH, int NT, int kWaves, bool A_LDS>
+int launch_kernel(const blkq4_gemm_args* a, int rows_log2) {
+  constexpr int kRedBytes = kWaves * NT * 64 * 4 * 4;
+  // the rows are copied 1 KiB at a time
+  const size_t lds_bytes = kRedBytes + (A_LDS ? ((((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023}) : 0);
+  auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, kWaves, A_LDS>;
+  static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
+  if (attr != hipSuccess) return static_cast<int>(attr);
+  hipLaunchKernelGGL(kernel, dim3((a->n / 16 + NT - 1) / NT), dim3(64 * kWaves), lds_bytes,
+                     static_cast<hipStream_t>(a->stream), static_cast<const uint16_t*>(a->a),
+                     static_cast<const uint4*>(a->packed_w), static_cast<const uint16_t*>(a->scales),
+                     static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c), a->m, a->n, a->k,
+                     rows_log2);
+  return static_cast<int>(hipGetLastError());
+}
+
+template <int BS, bool HAS_ZP, int DEPTH, int NT>
+int launch_waves(const blkq4_gemm_args* a) {
   // eight waves split K when there is enough of it: each wave has less to convert after its last
   // load has arrived, and more of that work overlaps the loads of the other waves
-  const int waves = (a->k >= 1024) ? 8 : 4;
-#define BLKQ4_LAUNCH_ZP(ZP_)                   \
-  if (nt == 1 && depth == 8) { BLKQ4_LAUNCH(ZP_, 8, 1); } \
-  else if (nt == 1) { BLKQ4_LAUNCH(ZP_, 4, 1); }   \
-  else if (nt == 2) { BLKQ4_LAUNCH(ZP_, 4, 2); }   \
-  else { BLKQ4_LAUNCH(ZP_, 4, 3); }
-  if (Z) { BLKQ4_LAUNCH_ZP(true); } else { BLKQ4_LAUNCH_ZP(false); }
-#undef BLKQ4_LAUNCH_ZP
-#undef BLKQ4_LAUNCH
-  return static_cast<int>(hipGetLastError());
+  int rows_log2 = 0;
+  while ((1 << rows_log2) < a->m) ++rows_log2;
+  const size_t a_bytes = (((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023};
+  if (a->k >= 4096 && BLKQ4_SKINNY_WAVES16) {
+    constexpr int kD = 2;
+    if (a_bytes + 16 * NT * 64 * 4 * 4 <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, kD, NT, 16, true>(a, rows_log2);
+    return launch_kernel<BS, HAS_ZP, kD, NT, 16, false>(a, rows_log2);
+  }
+  if (a->k >= 1024) {
+    constexpr int kD = DEPTH > 4 ? 4 : DEPTH;
+    if (a_bytes + 8 * NT * 64 * 4 * 4 <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, kD, NT, 8, true>(a, rows_log2);
+    return launch_kernel<BS, HAS_ZP, kD, NT, 8, false>(a, rows_log2);
+  }
+  return launch_kernel<BS, HAS_ZP, DEPTH, NT, 4, true>(a, rows_log2);  // K < 1024: at most 32 KiB of rows
+}
+
+template <int BS, bool HAS_ZP>
+int launch_shape(const blkq4_gemm_args* a) {
+  int nt, depth;
+  choose_shape(a->m, a->n, &nt, &depth);
+  if (nt == 1 && depth == 8) return launch_waves<BS, HAS_ZP, 8, 1>(a);
+  if (nt == 1) return launch_waves<BS, HAS_ZP, 4, 1>(a);
+  if (nt == 2) return launch_waves<BS, HAS_ZP, 4, 2>(a);
+  return launch_waves<BS, HAS_ZP, 4, 3>(a);
+}
+
+template <int BS>
+int launch_skinny(const blkq4_gemm_args* a) {
+  return a->zero_points ? launch_shape<BS, true>(a) : launch_shape<BS, false>(a);
 }
 
 }  // namespace
