@@ -52,6 +52,16 @@ constexpr int kBK = 64;
 
 // MFMA slot (0 .. slots-1) after which copy y of the range [lo, hi) is issued: evenly spread
 constexpr int copy_slot(int y, int lo, int hi, int slots) { return (hi > lo) ? (y - lo) * slots / (hi - lo) : -1; }
+// MFMA slot in whose shadow stage u of conversion pair g (of `pairs`) is issued.  Stages: 0 = both and-or,
+// 1 = first packed add, 2 = second packed add, 3 = both packed multiplies.  A pair has slots / pairs slots to
+// itself: with three or more the stages go and-or | adds | multiplies, with two and-or + add | add +
+// multiplies, with one everything in that order (dependent instructions are never adjacent).
+constexpr int stage_slot(int g, int u, int pairs, int slots) {
+  const int base = g * slots / pairs;
+  const int span = slots / pairs;
+  const int off = (span >= 3) ? ((u == 0) ? 0 : (u == 3) ? 2 : 1) : (span == 2) ? ((u <= 1) ? 0 : 1) : 0;
+  return (base + off < slots) ? base + off : slots - 1;
+}
 
 // Shape of a workgroup: WM x WN waves, each owning (32*RT) rows x (32*NT) columns (the WM waves of a
 // column group share its packed weights, scales and zero-points), plus PW producer waves that do
@@ -233,42 +243,51 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   block_barrier();
 
   // ---- LDS byte offsets of this lane's reads inside a stage ----
+  // (LDS addresses, so that a read costs one addition of the ring slot's offset and nothing else)
   uint32_t a_rd[4];  // activation fragment of step j, row tile 0 (row tile r is 4096 bytes further)
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    a_rd[j] = static_cast<uint32_t>(wm * (32 * RT) + i) * 128u + (((4 * h + j) ^ ((i >> 1) & 7)) * 16u);
+    a_rd[j] = lds0 + static_cast<uint32_t>(wm * (32 * RT) + i) * 128u + (((4 * h + j) ^ ((i >> 1) & 7)) * 16u);
   }
-  const uint32_t b_rd = St::kABytes + wn * (NT * 1024) + lane * 16;
-  const uint32_t m_rd = St::kABytes + St::kBBytes + wn * kBlocks * 256;
+  const uint32_t b_rd = lds0 + St::kABytes + wn * (NT * 1024) + lane * 16;
+  const uint32_t m_rd = lds0 + St::kABytes + St::kBBytes + wn * kBlocks * 256;
 
   const DequantMasks masks = DequantMasks::make();
 
-#define BLKQ4_READ_A1(dst_, stage_ptr_, j_, r_) \
-  (dst_)[r_] = as_half8(*reinterpret_cast<const uint4*>((stage_ptr_) + a_rd[j_] + (r_) * 4096))
+#define BLKQ4_READ_A1(dst_, stage_off_, j_, r_) (dst_)[r_] = as_half8(lds_read_16((stage_off_) + a_rd[j_], (r_) * 4096))
   // packed words, scales and zero-points of all the wave's fragments for one k tile
 #define BLKQ4_READ_B(words_, dc_, stage_ptr_)                                                \
   _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                           \
-    const uint4 u_ = *reinterpret_cast<const uint4*>((stage_ptr_) + b_rd + t * 1024);        \
+    const uint4 u_ = lds_read_16((stage_ptr_) + b_rd, t * 1024);                             \
     (words_)[t][0] = u_.x;                                                                   \
     (words_)[t][1] = u_.y;                                                                   \
     (words_)[t][2] = u_.z;                                                                   \
     (words_)[t][3] = u_.w;                                                                   \
     _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                      \
       const int blk_ = (BS == 64) ? 0 : (BS == 32) ? h : (2 * h + q);                        \
-      const uint8_t* mb_ = (stage_ptr_) + m_rd + (blk_ * 2 + t) * 128;                       \
-      (dc_##_sc)[t][q] = *reinterpret_cast<const uint16_t*>(mb_ + i * 2);                    \
-      (dc_##_zp)[t][q] = HAS_ZP ? static_cast<uint32_t>(mb_[64 + i]) : 8u;                   \
+      const uint32_t mb_ = (stage_ptr_) + m_rd + blk_ * 256;                                 \
+      (dc_##_sc)[t][q] = lds_read_u16(mb_ + i * 2, t * 128);                                 \
+      (dc_##_zp)[t][q] = HAS_ZP ? lds_read_u8(mb_ + i, t * 128 + 64) : 8u;                   \
     }                                                                                        \
   }
 #define BLKQ4_MAKE_CONSTS(dc_)                            \
   _Pragma("unroll") for (int t = 0; t < NT; ++t)          \
   _Pragma("unroll") for (int q = 0; q < kMeta; ++q)(dc_)[t][q] = make_dequant_consts((dc_##_sc)[t][q], (dc_##_zp)[t][q])
-  // piece x (0 .. 4*NT-1) of the conversion of word `w_` of every fragment into fragment buffer `dst_`:
-  // piece x is fp16 pair x % 4 of fragment x / 4
-#define BLKQ4_PIECE(dst_, words_, w_, dc_, q_, x_)                                                         \
-  wp[dst_][(x_) / 4][(x_) % 4] =                                                                           \
-      dequant_pair((((x_) % 4) >= 2) ? ((words_)[(x_) / 4][w_] >> 8) : (words_)[(x_) / 4][w_], (x_) % 4, \
-                   (dc_)[(x_) / 4][q_], masks)
+  // Piece y (0 .. 4*NT-1) of the conversion of word `w_` of every fragment into fragment buffer `dst_` is fp16
+  // pair y % 4 of fragment y / 4.  Its three instructions depend on each other (and a packed instruction
+  // that reads the result of the one before it costs a wait state), so two pieces are converted together,
+  // stage by stage: AO = v_and_or_b32, PA = v_pk_add_f16, PM = v_pk_mul_f16.
+#define BLKQ4_PIECE_AO(words_, w_, y_)                                                                     \
+  pt[y_] = as_half2((((((y_) % 4) >= 2) ? ((words_)[(y_) / 4][w_] >> 8) : (words_)[(y_) / 4][w_]) &      \
+                     ((((y_) & 1) == 0) ? masks.lo_mask : masks.hi_mask)) |                               \
+                    ((((y_) & 1) == 0) ? masks.magic_1024 : masks.magic_64))
+#define BLKQ4_PIECE_PA(dc_, q_, y_) \
+  pt[y_] = pt[y_] + ((((y_) & 1) == 0) ? (dc_)[(y_) / 4][q_].neg_c0 : (dc_)[(y_) / 4][q_].neg_c1)
+#define BLKQ4_PIECE_PM(dst_, dc_, q_, y_) wp[dst_][(y_) / 4][(y_) % 4] = pt[y_] * (dc_)[(y_) / 4][q_].scale2
+#define BLKQ4_PIECE(dst_, words_, w_, dc_, q_, y_) \
+  BLKQ4_PIECE_AO(words_, w_, y_);                  \
+  BLKQ4_PIECE_PA(dc_, q_, y_);                     \
+  BLKQ4_PIECE_PM(dst_, dc_, q_, y_)
 #define BLKQ4_WFRAG(slot_, t_) \
   __builtin_bit_cast(half8_t, half2x4_t{wp[slot_][t_][0], wp[slot_][t_][1], wp[slot_][t_][2], wp[slot_][t_][3]})
 
@@ -278,18 +297,21 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
 
   half8_t af[2][RT];      // activation fragments, double buffered over the k steps
   half2_t wp[2][NT][4];   // weight fragments (4 fp16 pairs each), double buffered
+  half2_t pt[4 * NT];     // pieces of a fragment on their way through the conversion
   uint32_t words[NT][4], nwords[NT][4];
   uint32_t dc_sc[NT][kMeta], dc_zp[NT][kMeta], ndc_sc[NT][kMeta], ndc_zp[NT][kMeta];
   DequantConsts dc[NT][kMeta], ndc[NT][kMeta];
 
   {
-    const uint8_t* s0 = lds;
+    const uint32_t s0 = 0;
     BLKQ4_READ_B(words, dc, s0);
     BLKQ4_MAKE_CONSTS(dc);
 #pragma unroll
     for (int r = 0; r < RT; ++r) BLKQ4_READ_A1(af[0], s0, 0, r);
 #pragma unroll
-    for (int x = 0; x < 4 * NT; ++x) BLKQ4_PIECE(0, words, 0, dc, 0, x);
+    for (int x = 0; x < 4 * NT; ++x) {
+      BLKQ4_PIECE(0, words, 0, dc, 0, x);
+    }
   }
 
   // One 16-deep k step: RT*NT MFMAs on fragment buffers `cur_`; in their shadow the LDS reads of the
@@ -305,8 +327,18 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
         const int x_ = r * NT + t;                                                                 \
         acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[t], af[cur_][r], acc[r][t], 0, 0, 0); \
         if (t == NT - 1) BLKQ4_READ_A1(af[1 - (cur_)], nstage_, nj_, r);                           \
-        _Pragma("unroll") for (int y = x_ * kPiecesPerMfma; y < (x_ + 1) * kPiecesPerMfma; ++y) {  \
-          if (y < 4 * NT) BLKQ4_PIECE(1 - (cur_), nwords_, nw_, ndc_, nq_, y);                     \
+        _Pragma("unroll") for (int g2 = 0; g2 < 2 * NT; ++g2) {                                    \
+          /* stage u of the pair's conversion is issued behind MFMA stage_slot(g2, u, ...) */      \
+          if (stage_slot(g2, 0, 2 * NT, kMfmas) == x_) {                                           \
+            BLKQ4_PIECE_AO(nwords_, nw_, 2 * g2);                                                  \
+            BLKQ4_PIECE_AO(nwords_, nw_, 2 * g2 + 1);                                              \
+          }                                                                                        \
+          if (stage_slot(g2, 1, 2 * NT, kMfmas) == x_) BLKQ4_PIECE_PA(ndc_, nq_, 2 * g2);          \
+          if (stage_slot(g2, 2, 2 * NT, kMfmas) == x_) BLKQ4_PIECE_PA(ndc_, nq_, 2 * g2 + 1);      \
+          if (stage_slot(g2, 3, 2 * NT, kMfmas) == x_) {                                           \
+            BLKQ4_PIECE_PM(1 - (cur_), ndc_, nq_, 2 * g2);                                         \
+            BLKQ4_PIECE_PM(1 - (cur_), ndc_, nq_, 2 * g2 + 1);                                     \
+          }                                                                                        \
         }                                                                                          \
         _Pragma("unroll") for (int y = (lo_); y < (hi_); ++y) {                                    \
           if (copy_slot(y, lo_, hi_, kMfmas) == x_) BLKQ4_COPY_OP(y, ctile_, cstage_);             \
@@ -315,7 +347,6 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
       }                                                                                            \
     }                                                                                              \
   }
-  constexpr int kPiecesPerMfma = (4 * NT + kMfmas - 1) / kMfmas;
   // The copies of one k tile are issued over the four steps that follow the barrier which frees
   // their ring slot (two steps when the ring has only three slots and the tile is needed sooner).
   constexpr int kCopySteps = (PW > 0) ? 0 : (kStages >= 4) ? 4 : 2;  // 0: the producer waves copy
@@ -325,8 +356,8 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
 
   for (int kt = 0; kt < KT; ++kt) {
     const int stage = kt % kStages;
-    const uint8_t* sa = lds + stage * St::kBytes;                         // tile kt
-    const uint8_t* sn = lds + ((kt + 1) % kStages) * St::kBytes;          // tile kt + 1
+    const uint32_t sa = stage * St::kBytes;                               // tile kt: offset of its ring slot
+    const uint32_t sn = ((kt + 1) % kStages) * St::kBytes;                // tile kt + 1
     const int copy_tile = min(kt + kDistance, KT - 1);                    // clamped: re-fetches the last tile
     const int copy_stage = (kt + kDistance) % kStages;
     const int late_tile = min(kt + kDistance - 1, KT - 1);                // the group begun in the previous tile
@@ -362,26 +393,49 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
 #undef BLKQ4_READ_B
 #undef BLKQ4_MAKE_CONSTS
 #undef BLKQ4_PIECE
+#undef BLKQ4_PIECE_AO
+#undef BLKQ4_PIECE_PA
+#undef BLKQ4_PIECE_PM
 #undef BLKQ4_WFRAG
 #undef BLKQ4_STEP
 
   // Epilogue.  Accumulator element 4*g + e of lane (i, h), fragment t, is output row m0 + 32*r + i and
-  // column nw0 + 32*t + 8*g + 4*h + e: four consecutive columns -> one 8-byte store.
+  // column nw0 + 32*t + 8*g + 4*h + e.  Stored straight from there, a wave's store instruction would touch
+  // 32 rows with 16 bytes each; instead every wave transposes its tile through a private piece of the
+  // (now unused) LDS ring, four row tiles at a time, and stores whole rows of its tile: 16 bytes per lane,
+  // 64*NT contiguous bytes per row.
+  block_barrier();  // nobody reads the ring any more
+  {
+    constexpr int kRowBytes = 64 * NT + 16;        // padded: consecutive rows start 4 (NT=2: 36) banks apart
+    constexpr int kPassTiles = (RT < 4) ? RT : 4;  // row tiles staged at a time
+    constexpr int kChunks = 4 * NT;                // 16-byte chunks per row
+    constexpr int kRowsPerStore = 64 / kChunks;
+    static_assert(kComputeWaves * 32 * kPassTiles * kRowBytes <= kStages * St::kBytes, "staging area does not fit");
+    const uint32_t region = lds0 + (wm * WN + wn) * (32 * kPassTiles * kRowBytes);
+    const int srow = lane / kChunks, chunk = lane % kChunks;
+    const int col = nw0 + chunk * 8;
 #pragma unroll
-  for (int r = 0; r < RT; ++r) {
-    const int m = m0 + wm * (32 * RT) + 32 * r + i;
-    if (m >= M) continue;
+    for (int r0 = 0; r0 < RT; r0 += kPassTiles) {
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      if (nw0 + 32 * t >= N) continue;
-      uint16_t* crow = C + static_cast<size_t>(m) * N + nw0 + 32 * t + 4 * h;
+      for (int r = r0; r < r0 + kPassTiles && r < RT; ++r) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const uint32_t lo = float_to_half_bits(acc[r][t][4 * g + 0]) |
-                            (static_cast<uint32_t>(float_to_half_bits(acc[r][t][4 * g + 1])) << 16);
-        const uint32_t hi = float_to_half_bits(acc[r][t][4 * g + 2]) |
-                            (static_cast<uint32_t>(float_to_half_bits(acc[r][t][4 * g + 3])) << 16);
-        *reinterpret_cast<uint2*>(crow + 8 * g) = make_uint2(lo, hi);
+        for (int t = 0; t < NT; ++t) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const uint32_t lo = float_to_half_bits(acc[r][t][4 * g + 0]) |
+                                (static_cast<uint32_t>(float_to_half_bits(acc[r][t][4 * g + 1])) << 16);
+            const uint32_t hi = float_to_half_bits(acc[r][t][4 * g + 2]) |
+                                (static_cast<uint32_t>(float_to_half_bits(acc[r][t][4 * g + 3])) << 16);
+            lds_write_8(region + ((r - r0) * 32 + i) * kRowBytes + h * 8, t * 64 + g * 16, lo, hi);
+          }
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < 32 * kPassTiles / kRowsPerStore; ++it) {
+        const int row = it * kRowsPerStore + srow;  // inside the pass
+        const uint4 v = lds_read_16(region + srow * kRowBytes + chunk * 16, it * kRowsPerStore * kRowBytes);
+        const int m = m0 + wm * (32 * RT) + r0 * 32 + row;
+        if (m < M && col < N) *reinterpret_cast<uint4*>(C + static_cast<size_t>(m) * N + col) = v;
       }
     }
   }

@@ -28,6 +28,27 @@ __device__ __forceinline__ void async_copy_4_flat_lo32(uint32_t lds_base, const 
       : "s"(lds_base), "v"(gptr)
       : "memory");
 }
+// LDS reads at byte address `addr` + `imm`.  `imm` is a compile-time constant applied as a pointer offset,
+// which the compiler folds into the instruction's offset field (it will not do that for an integer addition,
+// which may wrap); `addr` costs whatever the caller spends on it and nothing more.
+typedef uint32_t lds_u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 lds_read_16(uint32_t addr, int imm = 0) {
+  const auto* p = reinterpret_cast<const __attribute__((address_space(3))) uint8_t*>(addr) + imm;
+  const lds_u32x4_t v = *reinterpret_cast<const __attribute__((address_space(3))) lds_u32x4_t*>(p);
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ uint32_t lds_read_u16(uint32_t addr, int imm = 0) {
+  const auto* p = reinterpret_cast<const __attribute__((address_space(3))) uint8_t*>(addr) + imm;
+  return *reinterpret_cast<const __attribute__((address_space(3))) uint16_t*>(p);
+}
+__device__ __forceinline__ uint32_t lds_read_u8(uint32_t addr, int imm = 0) {
+  return *(reinterpret_cast<const __attribute__((address_space(3))) uint8_t*>(addr) + imm);
+}
+typedef uint32_t lds_u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void lds_write_8(uint32_t addr, int imm, uint32_t lo, uint32_t hi) {
+  auto* p = reinterpret_cast<__attribute__((address_space(3))) uint8_t*>(addr) + imm;
+  *reinterpret_cast<__attribute__((address_space(3))) lds_u32x2_t*>(p) = lds_u32x2_t{lo, hi};
+}
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
