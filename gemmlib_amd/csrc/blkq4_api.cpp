@@ -19,6 +19,12 @@ inline void set_error(std::string* err, std::string&& text) {
   if (err) *err = std::move(text);
 }
 
+// Which kernel multiplies m rows.  The reference switches at m > 16 (src/blkq4_f16_gemm_sm80.cu:343,
+// f16_gemm_sm80.h:63-72).  Here the weight-streaming kernel also takes 17..32 rows, and 33..64 rows while the
+// matrix is narrow: up to there it is faster than the tile kernel, whose grid cannot fill the chip when m is
+// that small (its time is flat in m and n, the streaming kernel's grows with both).
+inline bool streaming_kernel_takes(int m, int n) { return m <= 32 || (m <= 64 && n <= 6144); }
+
 inline bool supported_block_size(int bs) { return bs == 16 || bs == 32 || bs == 64; }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -235,8 +241,8 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
   args.stream = stream;
   // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
   const int code = !column_wise_blocking ? blkq4_dev_gemm_rowwise(&args)
-                   : (m > 16)            ? blkq4_dev_gemm(&args)
-                                         : blkq4_dev_skinny(&args);
+                   : streaming_kernel_takes(m, n) ? blkq4_dev_skinny(&args)
+                                                  : blkq4_dev_gemm(&args);
   if (code) return device_failure(code, err);
   return 0;
 }

@@ -69,7 +69,16 @@ WIDE_SKINNY_CASES = [
 ]
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES)
+# long K, where the activation rows no longer fit in LDS as a whole and are staged per k slice, and
+# 17..64 rows, which share one conversion of the weights between two or four row tiles
+LONG_K_CASES = [
+    (32, True, 16, 64, 8192 + 64), (64, False, 9, 64, 12288), (16, True, 3, 32, 40960 + 128),
+    (16, True, 32, 64, 4096), (32, True, 20, 96, 6144), (64, True, 64, 64, 4096), (32, False, 50, 96, 2112),
+    (64, True, 31, 4128, 320), (16, False, 64, 4128, 128), (32, True, 32, 8224, 2112), (16, True, 25, 8192 + 64, 4160),
+]
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + LONG_K_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
 
