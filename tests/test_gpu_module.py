@@ -70,3 +70,42 @@ def test_extension_argument_checks(device, mod):
         ext.forward(32, True, 64, 32, torch.zeros(4, 32, dtype=torch.float16, device=device), q_w, q_s, q_zp)
     with pytest.raises(RuntimeError, match="only supports float16 inputs"):
         ext.forward(32, True, 64, 32, torch.zeros(4, 64, device=device), q_w, q_s, q_zp)
+
+
+@pytest.mark.parametrize("col_wise", [True, False])
+def test_module_leading_dimensions_and_row_wise_blocks(oracle, device, mod, col_wise):
+    """[batch, seq, in_features] inputs, and the layer with quantization blocks along out_features."""
+    g = torch.Generator(device="cpu").manual_seed(11)
+    k, n, bs = 256, 192, 32
+    w = (torch.randn(n, k, generator=g) * 0.02).to(torch.float16)
+    x = torch.randn(3, 5, k, generator=g).to(torch.float16)
+    layer = mod.BlkQ4Linear(bs, col_wise, False, w.to(device))
+    y = layer(x.to(device))
+    assert y.shape == (3, 5, n)
+    w_np = w.view(torch.int16).numpy().view(np.float16)
+    canon, s, z = oracle.quantize(bs, col_wise, w_np, True)
+    ref = oracle.gemm(x.reshape(15, k).view(torch.int16).numpy().view(np.float16), oracle.dequantize(bs, col_wise, canon, s, z))
+    assert max_rel_err(to_np(y.reshape(15, n)), ref) <= 1e-2
+    assert torch.equal(layer(x.to(device).reshape(15, k)), y.reshape(15, n))
+
+
+def test_state_dict_round_trip_and_from_packed(device, mod):
+    g = torch.Generator(device="cpu").manual_seed(12)
+    k, n, bs = 128, 64, 64
+    w = (torch.randn(n, k, generator=g) * 0.02).to(torch.float16).to(device)
+    bias = torch.randn(n, generator=g).to(torch.float16).to(device)
+    x = torch.randn(7, k, generator=g).to(torch.float16).to(device)
+    layer = mod.BlkQ4Linear(bs, True, False, w, bias)
+    state = layer.state_dict()
+    assert {"q_weights", "q_scales", "q_zp", "bias"} <= set(state)
+    # a layer quantized from different weights takes over the saved tensors
+    other = mod.BlkQ4Linear(bs, True, False, torch.zeros_like(w), torch.zeros_like(bias))
+    other.load_state_dict(state)
+    assert torch.equal(other(x), layer(x))
+    # the quantization parameters are part of the state: a mismatching layer refuses it
+    with pytest.raises((ValueError, RuntimeError)):
+        mod.BlkQ4Linear(32, True, False, torch.zeros_like(w)).load_state_dict(state)
+    packed = mod.BlkQ4Linear.from_packed(bs, True, k, n, layer.q_weights, layer.q_scales, layer.q_zp, bias)
+    assert torch.equal(packed(x), layer(x))
+    with pytest.raises(ValueError):
+        mod.BlkQ4Linear.from_packed(bs, True, k, n + 32, layer.q_weights, layer.q_scales, layer.q_zp)
