@@ -20,10 +20,20 @@ inline void set_error(std::string* err, std::string&& text) {
 }
 
 // Which kernel multiplies m rows.  The reference switches at m > 16 (src/blkq4_f16_gemm_sm80.cu:343,
-// f16_gemm_sm80.h:63-72).  Here the weight-streaming kernel also takes 17..32 rows, and 33..64 rows while the
-// matrix is narrow: up to there it is faster than the tile kernel, whose grid cannot fill the chip when m is
-// that small (its time is flat in m and n, the streaming kernel's grows with both).
-inline bool streaming_kernel_takes(int m, int n) { return m <= 32 || (m <= 64 && n <= 6144); }
+// f16_gemm_sm80.h:63-72).  Here the weight-streaming kernel keeps going, in row groups of 32, for as long as
+// it is expected to be faster than the tile kernel, whose grid cannot fill the chip when m is small.
+// Both estimates are fits to measurements on MI355X: the streaming kernel's time grows with
+// row groups x n x k (2.8 us per row group at n = k = 4096), the tile kernel runs its k / 64 steps of 0.64 us
+// once per round of 256 workgroups of 128 x 256 outputs.
+inline bool streaming_kernel_takes(int m, int n, int k) {
+  if (m <= 32) return true;
+  if (m > 1024) return false;
+  const double row_groups = (m + 31) / 32;
+  const double streaming_us = 2.8 * row_groups * (static_cast<double>(n) / 4096.0) * (static_cast<double>(k) / 4096.0);
+  const long workgroups = static_cast<long>((m + 127) / 128) * ((n + 255) / 256);
+  const double tile_us = static_cast<double>((workgroups + 255) / 256) * (k / 64) * 0.64;
+  return streaming_us < tile_us;
+}
 
 inline bool supported_block_size(int bs) { return bs == 16 || bs == 32 || bs == 64; }
 
@@ -241,7 +251,7 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
   args.stream = stream;
   // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
   const int code = !column_wise_blocking ? blkq4_dev_gemm_rowwise(&args)
-                   : streaming_kernel_takes(m, n) ? blkq4_dev_skinny(&args)
+                   : streaming_kernel_takes(m, n, k) ? blkq4_dev_skinny(&args)
                                                   : blkq4_dev_gemm(&args);
   if (code) return device_failure(code, err);
   return 0;

@@ -57,17 +57,30 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
                                                                const uint4* __restrict__ W,
                                                                const uint16_t* __restrict__ S,
                                                                const uint8_t* __restrict__ Z,
-                                                               uint16_t* __restrict__ C, int M, int N,
-                                                               int K, int rows_log2) {
+                                                               uint16_t* __restrict__ C, int M_total, int N,
+                                                               int K, int rows_log2, int row_groups) {
   constexpr int kMeta = Slot<BS, NT, MT, AM>::kMeta;
   constexpr bool A_LDS = AM == kRowsWholeInLds;
   constexpr int kLoads = NT * (1 + kMeta * (HAS_ZP ? 2 : 1));  // weight / scale / zero-point requests of a slot
   constexpr int kSlotRows = 16 * MT;                           // kRowsPerSlotInLds: rows staged per slot
   constexpr int kSlotBytes = kSlotRows * 256;
-  constexpr int kRedFloats = kWaves * NT * MT * 64 * 4;
+  // the partial tiles of the final reduction reuse the LDS of the activation rows
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   float* red = reinterpret_cast<float*>(smem);
-  const uint8_t* a_lds = smem + kRedFloats * 4;
+  const uint8_t* a_lds = smem;
+
+  // Workgroup -> (row group of 16 * MT rows, group of NT column tiles).  Consecutive workgroups go to
+  // consecutive XCDs; the row groups of one column group are 8 apart, so they run on the same XCD and the
+  // weights they share stay in that XCD's L2.
+  const int col_groups = ((N >> 4) + NT - 1) / NT;
+  const int wg = blockIdx.x;
+  const int rg = (wg >> 3) % row_groups;
+  const int cg = (wg & 7) + 8 * ((wg >> 3) / row_groups);
+  if (cg >= col_groups) return;  // the grid is rounded up to whole groups of 8
+  const int m0 = rg * (16 * MT);
+  const int M = min(16 * MT, M_total - m0);
+  A += static_cast<size_t>(m0) * K;
+  C += static_cast<size_t>(m0) * N;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -80,8 +93,8 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   int n[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int tile = blockIdx.x * NT + t;
-    n[t] = ((tile < tiles) ? tile : blockIdx.x * NT) * 16 + nl;
+    const int tile = cg * NT + t;
+    n[t] = ((tile < tiles) ? tile : cg * NT) * 16 + nl;
   }
   const DequantMasks masks = DequantMasks::make();
   // lanes without a row (past M) re-read the last row: an output element depends on its own activation
@@ -110,7 +123,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   uint32_t a_rd = 0;  // LDS byte offset of this lane's row inside a unit, chunk 0
   uint32_t a_swz = 0;
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
-                            (__attribute__((address_space(3))) uint8_t*)(smem))) + kRedFloats * 4;
+                            (__attribute__((address_space(3))) uint8_t*)(smem)));
   if (AM == kRowsPerSlotInLds) {
     // this wave's slots: DEPTH pieces of [4 units][kSlotRows rows][64 B]
     a_rd = (wave * DEPTH) * kSlotBytes + g * (kSlotRows * 64) + nl * 64;
@@ -237,7 +250,8 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   }
 #undef BLKQ4_LOAD_SLOT
 
-  // cross-wave reduction through LDS
+  // cross-wave reduction through LDS (which holds activation rows until every wave is done with them)
+  if (AM != kRowsInRegisters) __syncthreads();
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -253,8 +267,8 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     for (int w = 0; w < kWaves; ++w) r += red[w * (NT * MT * 256) + v];
     const int t = v / (MT * 256), mt = (v >> 8) % MT, L = (v >> 2) & 63, e = v & 3;
     const int row = 16 * mt + (L & 15);
-    if (row < M && blockIdx.x * NT + t < tiles) {
-      C[static_cast<size_t>(row) * N + blockIdx.x * (16 * NT) + 16 * t + 4 * (L >> 4) + e] = float_to_half_bits(r);
+    if (row < M && cg * NT + t < tiles) {
+      C[static_cast<size_t>(row) * N + cg * (16 * NT) + 16 * t + 4 * (L >> 4) + e] = float_to_half_bits(r);
     }
   }
 }
@@ -264,9 +278,8 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 // unit works through ceil(workgroups / 256) * T tiles.  Wider workgroups also re-read the activation
 // rows less often, which weighs more the more rows there are.
 constexpr size_t kMaxLdsBytes = 160 * 1024;
-#ifndef BLKQ4_SKINNY_WAVES16
-#define BLKQ4_SKINNY_WAVES16 1
-#endif
+constexpr int kStreamingMaxRows = 1024;
+
 
 void choose_shape(int m, int n, int* nt, int* depth) {
   constexpr int kComputeUnits = 256;
@@ -288,77 +301,72 @@ void choose_shape(int m, int n, int* nt, int* depth) {
   *depth = (*nt == 1 && tiles <= 2 * kComputeUnits) ? 8 : 4;
 }
 
-// One kernel instantiation: raises its dynamic-LDS limit once, then launches.
+// One kernel instantiation: raises its dynamic-LDS limit once, then launches `row_groups` row groups of
+// 16 * MT rows each.
 template <int BS, bool HAS_ZP, int DEPTH, int NT, int MT, int kWaves, int AM>
-int launch_kernel(const blkq4_gemm_args* a, int rows_log2) {
-  constexpr int kRedBytes = kWaves * NT * MT * 64 * 4 * 4;
+int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
+  constexpr size_t kRedBytes = static_cast<size_t>(kWaves) * NT * MT * 64 * 4 * 4;
   constexpr size_t kPerSlotBytes = static_cast<size_t>(kWaves) * DEPTH * 16 * MT * 256;
-  static_assert(AM != kRowsPerSlotInLds || kRedBytes + kPerSlotBytes <= kMaxLdsBytes, "slots do not fit in LDS");
-  // the rows are copied 1 KiB at a time
-  const size_t lds_bytes =
-      kRedBytes + (AM == kRowsWholeInLds ? ((((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023})
-                   : AM == kRowsPerSlotInLds ? kPerSlotBytes
-                                             : 0);
+  static_assert(kRedBytes <= kMaxLdsBytes, "partial tiles do not fit in LDS");
+  static_assert(AM != kRowsPerSlotInLds || kPerSlotBytes <= kMaxLdsBytes, "slots do not fit in LDS");
+  // the rows are copied 1 KiB at a time; the partial tiles of the reduction reuse their space
+  const size_t a_bytes = AM == kRowsWholeInLds ? ((((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023})
+                         : AM == kRowsPerSlotInLds ? kPerSlotBytes
+                                                   : 0;
+  const size_t lds_bytes = a_bytes > kRedBytes ? a_bytes : kRedBytes;
   auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM>;
   static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
   if (attr != hipSuccess) return static_cast<int>(attr);
-  hipLaunchKernelGGL(kernel, dim3((a->n / 16 + NT - 1) / NT), dim3(64 * kWaves), lds_bytes,
-                     static_cast<hipStream_t>(a->stream), static_cast<const uint16_t*>(a->a),
-                     static_cast<const uint4*>(a->packed_w), static_cast<const uint16_t*>(a->scales),
-                     static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c), a->m, a->n, a->k,
-                     rows_log2);
+  const int col_groups = (a->n / 16 + NT - 1) / NT;
+  const unsigned grid = static_cast<unsigned>((col_groups + 7) / 8) * 8u * static_cast<unsigned>(row_groups);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * kWaves), lds_bytes, static_cast<hipStream_t>(a->stream),
+                     static_cast<const uint16_t*>(a->a), static_cast<const uint4*>(a->packed_w),
+                     static_cast<const uint16_t*>(a->scales), static_cast<const uint8_t*>(a->zero_points),
+                     static_cast<uint16_t*>(a->c), a->m, a->n, a->k, rows_log2, row_groups);
   return static_cast<int>(hipGetLastError());
 }
 
+// M <= 16: one row tile; the waves of a workgroup split K.
 template <int BS, bool HAS_ZP, int DEPTH, int NT>
 int launch_waves(const blkq4_gemm_args* a) {
-  // eight waves split K when there is enough of it: each wave has less to convert after its last
-  // load has arrived, and more of that work overlaps the loads of the other waves
   int rows_log2 = 0;
   while ((1 << rows_log2) < a->m) ++rows_log2;
   const size_t a_bytes = (((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023};
-  if (a->k >= 4096 && BLKQ4_SKINNY_WAVES16) {
-    constexpr int kD = 2;
-    if (a_bytes + 16 * NT * 64 * 4 * 4 <= kMaxLdsBytes) {
-      return launch_kernel<BS, HAS_ZP, kD, NT, 1, 16, kRowsWholeInLds>(a, rows_log2);
-    }
+  // sixteen waves when there is enough K: each wave has less to convert after its last load has arrived,
+  // and more of that work overlaps the loads of the other waves
+  if (a->k >= 4096 && a_bytes <= kMaxLdsBytes) {
+    return launch_kernel<BS, HAS_ZP, 2, NT, 1, 16, kRowsWholeInLds>(a, rows_log2);
   }
   if (a->k >= 1024) {
     constexpr int kD = DEPTH > 4 ? 4 : DEPTH;
-    if (a_bytes + 8 * NT * 64 * 4 * 4 <= kMaxLdsBytes) {
-      return launch_kernel<BS, HAS_ZP, kD, NT, 1, 8, kRowsWholeInLds>(a, rows_log2);
-    }
+    if (a_bytes <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, kD, NT, 1, 8, kRowsWholeInLds>(a, rows_log2);
     return launch_kernel<BS, HAS_ZP, kD, NT, 1, 8, kRowsPerSlotInLds>(a, rows_log2);  // 8 * 4 * 4 KiB of rows
   }
   return launch_kernel<BS, HAS_ZP, DEPTH, NT, 1, 4, kRowsWholeInLds>(a, rows_log2);  // K < 1024: at most 32 KiB of rows
 }
 
-// 16 < M <= 16 * MT: one conversion of the weights feeds MT row tiles; eight waves, NT column tiles.
-template <int BS, bool HAS_ZP, int MT, int NT>
-int launch_rows_nt(const blkq4_gemm_args* a) {
-  int rows_log2 = 0;
-  while ((1 << rows_log2) < a->m) ++rows_log2;
-  const size_t a_bytes = (((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023};
-  if (a_bytes + 8 * NT * MT * 64 * 4 * 4 <= kMaxLdsBytes) {
-    return launch_kernel<BS, HAS_ZP, 2, NT, MT, 8, kRowsWholeInLds>(a, rows_log2);
-  }
-  // 8 waves x 2 slots x 8 KiB of rows fit for 32 rows; 64 rows go through registers
-  return launch_kernel<BS, HAS_ZP, 2, NT, MT, 8, (MT <= 2) ? kRowsPerSlotInLds : kRowsInRegisters>(a, rows_log2);
-}
-
-template <int BS, bool HAS_ZP, int MT>
-int launch_rows(const blkq4_gemm_args* a) {
-  // every workgroup fetches all the rows; two column tiles per workgroup halve that traffic as soon as
-  // there are enough tiles for every compute unit to get a workgroup all the same
-  if (MT == 2 && a->n / 16 >= 512) return launch_rows_nt<BS, HAS_ZP, MT, (MT == 2) ? 2 : 1>(a);
-  return launch_rows_nt<BS, HAS_ZP, MT, 1>(a);
+// M > 16: row groups of 32 rows (two row tiles share one conversion of the weights), NT column tiles per
+// workgroup, eight waves.
+template <int BS, bool HAS_ZP, int NT>
+int launch_rows(const blkq4_gemm_args* a, int row_groups) {
+  const size_t a_bytes = static_cast<size_t>(a->k) * 2 * 32;
+  if (a_bytes <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, 2, NT, 2, 8, kRowsWholeInLds>(a, 5, row_groups);
+  return launch_kernel<BS, HAS_ZP, 2, NT, 2, 8, kRowsPerSlotInLds>(a, 5, row_groups);  // 8 * 2 * 8 KiB of rows
 }
 
 template <int BS, bool HAS_ZP>
 int launch_shape(const blkq4_gemm_args* a) {
-  if (a->m > 32) return launch_rows<BS, HAS_ZP, 4>(a);
-  if (a->m > 16) return launch_rows<BS, HAS_ZP, 2>(a);
+  if (a->m > 16) {
+    // Every workgroup fetches the 32 rows of its group for all of K, so wide workgroups (more column tiles)
+    // mean less activation traffic; but there should be a workgroup for every compute unit.
+    constexpr int kComputeUnits = 256;
+    const int row_groups = (a->m + 31) / 32;
+    const long tiles = static_cast<long>(a->n / 16) * row_groups;
+    if (tiles >= 4 * kComputeUnits) return launch_rows<BS, HAS_ZP, 4>(a, row_groups);
+    if (tiles >= 2 * kComputeUnits) return launch_rows<BS, HAS_ZP, 2>(a, row_groups);
+    return launch_rows<BS, HAS_ZP, 1>(a, row_groups);
+  }
   int nt, depth;
   choose_shape(a->m, a->n, &nt, &depth);
   if (nt == 1 && depth == 8) return launch_waves<BS, HAS_ZP, 8, 1>(a);
@@ -375,7 +383,7 @@ int launch_skinny(const blkq4_gemm_args* a) {
 }  // namespace
 
 extern "C" int blkq4_dev_skinny(const blkq4_gemm_args* a) {
-  if (a->m < 1 || a->m > 64 || (a->n % 16) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
+  if (a->m < 1 || a->m > kStreamingMaxRows || (a->n % 16) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
   switch (a->block_size) {
     case 16: return launch_skinny<16>(a);
     case 32: return launch_skinny<32>(a);

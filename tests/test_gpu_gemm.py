@@ -70,11 +70,13 @@ WIDE_SKINNY_CASES = [
 
 
 # long K, where the activation rows no longer fit in LDS as a whole and are staged per k slice, and
-# 17..64 rows, which share one conversion of the weights between two or four row tiles
+# more than 16 rows in the streaming kernel: row groups of 32 rows (two row tiles share one conversion of
+# the weights), one, two or four column tiles per workgroup
 LONG_K_CASES = [
     (32, True, 16, 64, 8192 + 64), (64, False, 9, 64, 12288), (16, True, 3, 32, 40960 + 128),
     (16, True, 32, 64, 4096), (32, True, 20, 96, 6144), (64, True, 64, 64, 4096), (32, False, 50, 96, 2112),
     (64, True, 31, 4128, 320), (16, False, 64, 4128, 128), (32, True, 32, 8224, 2112), (16, True, 25, 8192 + 64, 4160),
+    (64, True, 100, 96, 8256), (16, True, 77, 4128, 192), (32, False, 130, 4128, 128), (64, False, 250, 1056, 320),
 ]
 
 
