@@ -23,15 +23,18 @@ inline void set_error(std::string* err, std::string&& text) {
 // f16_gemm_sm80.h:63-72).  Here the weight-streaming kernel keeps going, in row groups of 32, for as long as
 // it is expected to be faster than the tile kernel, whose grid cannot fill the chip when m is small.
 // Both estimates are fits to measurements on MI355X: the streaming kernel's time grows with
-// row groups x n x k (2.8 us per row group at n = k = 4096), the tile kernel runs its k / 64 steps of 0.64 us
-// once per round of 256 workgroups of 128 x 256 outputs.
+// row groups x n x k (2.8 us per row group at n = k = 4096); the tile kernel runs its k / 64 steps once per
+// round of 256 workgroups, 0.64 us a step with 128 x 256 tiles and 0.42 us with the 128 x 128 tiles it uses
+// when those cover the problem in one round.
 inline bool streaming_kernel_takes(int m, int n, int k) {
   if (m <= 32) return true;
   if (m > 1024) return false;
   const double row_groups = (m + 31) / 32;
   const double streaming_us = 2.8 * row_groups * (static_cast<double>(n) / 4096.0) * (static_cast<double>(k) / 4096.0);
+  const long small_tiles = static_cast<long>((m + 127) / 128) * ((n + 127) / 128);
   const long workgroups = static_cast<long>((m + 127) / 128) * ((n + 255) / 256);
-  const double tile_us = static_cast<double>((workgroups + 255) / 256) * (k / 64) * 0.64;
+  const double tile_us = (small_tiles <= 256) ? (k / 64) * 0.42
+                                              : static_cast<double>((workgroups + 255) / 256) * (k / 64) * 0.64;
   return streaming_us < tile_us;
 }
 
