@@ -26,7 +26,8 @@ inline void set_error(std::string* err, std::string&& text) {
 // row groups x n x k (2.8 us per row group at n = k = 4096); the tile kernel runs its k / 64 steps once per
 // round of 256 workgroups, 0.64 us a step with 128 x 256 tiles and 0.42 us with the 128 x 128 tiles it uses
 // when those cover the problem in one round.
-inline bool streaming_kernel_takes(int m, int n, int k) {
+inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k) {
+  if (!column_wise) return m <= 384;  // blocks along N: the tile kernel for them is a plain one (K=N=4096: 99 us at m = 256)
   if (m <= 32) return true;
   if (m > 1024) return false;
   const double row_groups = (m + 31) / 32;
@@ -253,9 +254,9 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
   args.c = output_ptr;
   args.stream = stream;
   // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
-  const int code = !column_wise_blocking ? blkq4_dev_gemm_rowwise(&args)
-                   : streaming_kernel_takes(m, n, k) ? blkq4_dev_skinny(&args)
-                                                  : blkq4_dev_gemm(&args);
+  const int code = streaming_kernel_takes(column_wise_blocking, m, n, k) ? blkq4_dev_skinny(&args)
+                   : column_wise_blocking                                ? blkq4_dev_gemm(&args)
+                                                                         : blkq4_dev_gemm_rowwise(&args);
   if (code) return device_failure(code, err);
   return 0;
 }

@@ -38,12 +38,16 @@ constexpr int kRowsInRegisters = 0;  // each lane loads its rows' 64 bytes per s
 constexpr int kRowsWholeInLds = 1;   // all rows, all of K, staged once per workgroup
 constexpr int kRowsPerSlotInLds = 2; // 16 * MT rows x 128 k staged per slot, private to the wave
 
-template <int BS, int NT, int MT, int AM>
+template <int BS, int NT, int MT, int AM, bool ROW>
 struct Slot {
   static constexpr int kMeta = (BS == 16) ? 2 : 1;  // quantization blocks inside one 32-deep unit
   uint4 w[NT];
-  uint32_t sc[NT][kMeta];
-  uint32_t zp[NT][kMeta];
+  uint32_t sc[NT][ROW ? 1 : kMeta];
+  uint32_t zp[NT][ROW ? 1 : kMeta];
+  // blocks along N: a scale and a zero-point per k, 32 of each for the lane's unit, in the packed order of
+  // the meta data (two 16-row groups of 32 + 16 bytes)
+  uint4 rs[ROW ? NT : 1][4];
+  uint4 rz[ROW ? NT : 1][2];
   uint4 a[AM == kRowsInRegisters ? 4 * MT : 1];  // 32 k of this lane's activation rows (unused when they are in LDS)
 };
 
@@ -52,16 +56,19 @@ struct Slot {
 // weights.  AM: where the activation rows are (see above).  kRowsWholeInLds: rows_log2 = log2 of the number
 // of rows kept in LDS, a power of two >= M, and the dynamic LDS size is red_bytes + (K * 2 << rows_log2).
 // kRowsPerSlotInLds: red_bytes + kWaves * DEPTH * 16 * MT * 256.
-template <int BS, bool HAS_ZP, int DEPTH, int NT, int MT, int kWaves, int AM>
+// ROW: quantization blocks run along N (one k, BS columns); S and Z are then in the packed order
+// described in blkq4_device.h and the lane's column group decides which 64 + 32 bytes it fetches per unit.
+template <int BS, bool HAS_ZP, int DEPTH, int NT, int MT, int kWaves, int AM, bool ROW>
 __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t* __restrict__ A,
                                                                const uint4* __restrict__ W,
                                                                const uint16_t* __restrict__ S,
                                                                const uint8_t* __restrict__ Z,
                                                                uint16_t* __restrict__ C, int M_total, int N,
                                                                int K, int rows_log2, int row_groups) {
-  constexpr int kMeta = Slot<BS, NT, MT, AM>::kMeta;
+  constexpr int kMeta = Slot<BS, NT, MT, AM, ROW>::kMeta;
   constexpr bool A_LDS = AM == kRowsWholeInLds;
-  constexpr int kLoads = NT * (1 + kMeta * (HAS_ZP ? 2 : 1));  // weight / scale / zero-point requests of a slot
+  // weight / scale / zero-point requests of a slot
+  constexpr int kLoads = ROW ? NT * (1 + 4 + (HAS_ZP ? 2 : 0)) : NT * (1 + kMeta * (HAS_ZP ? 2 : 1));
   constexpr int kSlotRows = 16 * MT;                           // kRowsPerSlotInLds: rows staged per slot
   constexpr int kSlotBytes = kSlotRows * 256;
   // the partial tiles of the final reduction reuse the LDS of the activation rows
@@ -116,7 +123,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
-  Slot<BS, NT, MT, AM> slot[DEPTH];
+  Slot<BS, NT, MT, AM, ROW> slot[DEPTH];
 
   // Rows to LDS: copy q fills LDS bytes [1024 q, 1024 q + 1024) of the [unit][row][64 B] layout, lane l
   // the 16 bytes at 16 l.  They are requested before anything else, so every later wait covers them.
@@ -151,6 +158,9 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     const bool ok_ = ks_ < units;                                                              \
     const int ksg_ = ok_ ? ks_ : (ks_ & wrap_mask);                                            \
     const int b_ = (BS == 64) ? (ksg_ >> 1) : (BS == 32) ? ksg_ : (2 * ksg_);                  \
+    /* the scales of a slice past the end are zeroed with a mask, not a select: a select lets the   */ \
+    /* compiler skip the load, and the waits below count every load of a slot                       */ \
+    const uint32_t okm_ = ok_ ? 0xffffffffu : 0u;                                              \
     if (AM == kRowsPerSlotInLds) {                                                             \
       /* copy q: LDS bytes [1024 q, 1024 q + 1024) of the slot, lane l the 16 bytes at 16 l; */ \
       /* requested before the slot's weights, so whoever has the weights has the rows        */ \
@@ -166,11 +176,24 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     }                                                                                          \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                           \
       (dst_).w[t] = W[static_cast<size_t>(ksg_) * N + n[t]];                                  \
-      _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                      \
-        const size_t mi_ = static_cast<size_t>(b_ + q) * N + n[t];                           \
-        const uint32_t sc_ = S[mi_];                                                           \
-        (dst_).sc[t][q] = ok_ ? sc_ : 0u;                                                      \
-        (dst_).zp[t][q] = HAS_ZP ? static_cast<uint32_t>(Z[mi_]) : 8u;                         \
+      if (ROW) {                                                                               \
+        const size_t mi_ = static_cast<size_t>(n[t] / BS) * K + static_cast<size_t>(ksg_) * 32; \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                        \
+          const uint4 v_ = reinterpret_cast<const uint4*>(S + mi_)[q];                         \
+          (dst_).rs[ROW ? t : 0][q] = make_uint4(v_.x & okm_, v_.y & okm_, v_.z & okm_, v_.w & okm_); \
+        }                                                                                      \
+        if (HAS_ZP) {                                                                          \
+          _Pragma("unroll") for (int q = 0; q < 2; ++q) {                                      \
+            (dst_).rz[ROW ? t : 0][q] = reinterpret_cast<const uint4*>(Z + mi_)[q];            \
+          }                                                                                    \
+        }                                                                                      \
+      } else {                                                                                 \
+        _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                    \
+          const size_t mi_ = static_cast<size_t>(b_ + q) * N + n[t];                         \
+          const uint32_t sc_ = S[mi_];                                                         \
+          (dst_).sc[t][ROW ? 0 : q] = sc_ & okm_;                                              \
+          (dst_).zp[t][ROW ? 0 : q] = HAS_ZP ? static_cast<uint32_t>(Z[mi_]) : 8u;             \
+        }                                                                                      \
       }                                                                                        \
     }                                                                                          \
     if (AM == kRowsInRegisters) {                                                              \
@@ -226,19 +249,46 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       }
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        DequantConsts dc[kMeta];
-#pragma unroll
-        for (int q = 0; q < kMeta; ++q) dc[q] = make_dequant_consts(slot[d].sc[t][q], slot[d].zp[t][q]);
         const uint32_t words[4] = {slot[d].w[t].x, slot[d].w[t].y, slot[d].w[t].z, slot[d].w[t].w};
+        DequantConsts dc[kMeta];
+        if (!ROW) {
+#pragma unroll
+          for (int q = 0; q < kMeta; ++q) dc[q] = make_dequant_consts(slot[d].sc[t][ROW ? 0 : q], slot[d].zp[t][ROW ? 0 : q]);
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const DequantConsts& c = dc[(kMeta == 2) ? (j >> 1) : 0];
           const uint32_t y = words[j] >> 8;
-          const half2_t p0 = dequant_pair(words[j], 0, c, masks), p1 = dequant_pair(words[j], 1, c, masks);
-          const half2_t p2 = dequant_pair(y, 2, c, masks), p3 = dequant_pair(y, 3, c, masks);
+          half2_t p[4];
+          if (ROW) {
+            // word j is rows 8 hh .. 8 hh + 7 of 16-row group j / 2 of the unit: pair i has its scales in
+            // 32-bit word 2 i + hh of the group and its zero-points in byte pair hh of word i
+            constexpr int kRowSlot = ROW ? 1 : 0;
+            const int hh = j & 1;
+            const uint4 s0 = slot[d].rs[kRowSlot * t][2 * (j >> 1)], s1 = slot[d].rs[kRowSlot * t][2 * (j >> 1) + 1];
+            const uint32_t sw[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+            const uint4 zq = HAS_ZP ? slot[d].rz[kRowSlot * t][j >> 1] : make_uint4(0, 0, 0, 0);
+            const uint32_t zw[4] = {zq.x, zq.y, zq.z, zq.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const uint32_t zpair = HAS_ZP ? ((zw[i] >> (8 * hh)) & 0x00ff00ffu) : 0x00080008u;
+              const uint32_t src = (i >= 2) ? y : words[j];
+              const half2_t s2 = as_half2(sw[2 * i + hh]);
+              if ((i & 1) == 0) {
+                p[i] = (as_half2((src & masks.lo_mask) | masks.magic_1024) + as_half2(0xE400E400u | zpair)) * s2;
+              } else {
+                p[i] = (as_half2((src & masks.hi_mask) | masks.magic_64) + as_half2(0xD400D400u | (zpair << 4))) * s2;
+              }
+            }
+          } else {
+            const DequantConsts& c = dc[(kMeta == 2) ? (j >> 1) : 0];
+            p[0] = dequant_pair(words[j], 0, c, masks);
+            p[1] = dequant_pair(words[j], 1, c, masks);
+            p[2] = dequant_pair(y, 2, c, masks);
+            p[3] = dequant_pair(y, 3, c, masks);
+          }
           half8_t wf;
-          wf[0] = p0[0]; wf[1] = p0[1]; wf[2] = p1[0]; wf[3] = p1[1];
-          wf[4] = p2[0]; wf[5] = p2[1]; wf[6] = p3[0]; wf[7] = p3[1];
+          wf[0] = p[0][0]; wf[1] = p[0][1]; wf[2] = p[1][0]; wf[3] = p[1][1];
+          wf[4] = p[2][0]; wf[5] = p[2][1]; wf[6] = p[3][0]; wf[7] = p[3][1];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
             acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, af[mt][j], acc[t][mt], 0, 0, 0);
@@ -303,7 +353,7 @@ void choose_shape(int m, int n, int* nt, int* depth) {
 
 // One kernel instantiation: raises its dynamic-LDS limit once, then launches `row_groups` row groups of
 // 16 * MT rows each.
-template <int BS, bool HAS_ZP, int DEPTH, int NT, int MT, int kWaves, int AM>
+template <int BS, bool HAS_ZP, bool ROW, int DEPTH, int NT, int MT, int kWaves, int AM>
 int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
   constexpr size_t kRedBytes = static_cast<size_t>(kWaves) * NT * MT * 64 * 4 * 4;
   constexpr size_t kPerSlotBytes = static_cast<size_t>(kWaves) * DEPTH * 16 * MT * 256;
@@ -314,7 +364,7 @@ int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
                          : AM == kRowsPerSlotInLds ? kPerSlotBytes
                                                    : 0;
   const size_t lds_bytes = a_bytes > kRedBytes ? a_bytes : kRedBytes;
-  auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM>;
+  auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW>;
   static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
   if (attr != hipSuccess) return static_cast<int>(attr);
@@ -328,7 +378,7 @@ int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
 }
 
 // M <= 16: one row tile; the waves of a workgroup split K.
-template <int BS, bool HAS_ZP, int DEPTH, int NT>
+template <int BS, bool HAS_ZP, bool ROW, int DEPTH, int NT>
 int launch_waves(const blkq4_gemm_args* a) {
   int rows_log2 = 0;
   while ((1 << rows_log2) < a->m) ++rows_log2;
@@ -336,26 +386,26 @@ int launch_waves(const blkq4_gemm_args* a) {
   // sixteen waves when there is enough K: each wave has less to convert after its last load has arrived,
   // and more of that work overlaps the loads of the other waves
   if (a->k >= 4096 && a_bytes <= kMaxLdsBytes) {
-    return launch_kernel<BS, HAS_ZP, 2, NT, 1, 16, kRowsWholeInLds>(a, rows_log2);
+    return launch_kernel<BS, HAS_ZP, ROW, 2, NT, 1, 16, kRowsWholeInLds>(a, rows_log2);
   }
   if (a->k >= 1024) {
     constexpr int kD = DEPTH > 4 ? 4 : DEPTH;
-    if (a_bytes <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, kD, NT, 1, 8, kRowsWholeInLds>(a, rows_log2);
-    return launch_kernel<BS, HAS_ZP, kD, NT, 1, 8, kRowsPerSlotInLds>(a, rows_log2);  // 8 * 4 * 4 KiB of rows
+    if (a_bytes <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, ROW, kD, NT, 1, 8, kRowsWholeInLds>(a, rows_log2);
+    return launch_kernel<BS, HAS_ZP, ROW, kD, NT, 1, 8, kRowsPerSlotInLds>(a, rows_log2);  // 8 * 4 * 4 KiB of rows
   }
-  return launch_kernel<BS, HAS_ZP, DEPTH, NT, 1, 4, kRowsWholeInLds>(a, rows_log2);  // K < 1024: at most 32 KiB of rows
+  return launch_kernel<BS, HAS_ZP, ROW, DEPTH, NT, 1, 4, kRowsWholeInLds>(a, rows_log2);  // K < 1024: at most 32 KiB of rows
 }
 
 // M > 16: row groups of 32 rows (two row tiles share one conversion of the weights), NT column tiles per
 // workgroup, eight waves.
-template <int BS, bool HAS_ZP, int NT>
+template <int BS, bool HAS_ZP, bool ROW, int NT>
 int launch_rows(const blkq4_gemm_args* a, int row_groups) {
   const size_t a_bytes = static_cast<size_t>(a->k) * 2 * 32;
-  if (a_bytes <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, 2, NT, 2, 8, kRowsWholeInLds>(a, 5, row_groups);
-  return launch_kernel<BS, HAS_ZP, 2, NT, 2, 8, kRowsPerSlotInLds>(a, 5, row_groups);  // 8 * 2 * 8 KiB of rows
+  if (a_bytes <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, ROW, 2, NT, 2, 8, kRowsWholeInLds>(a, 5, row_groups);
+  return launch_kernel<BS, HAS_ZP, ROW, 2, NT, 2, 8, kRowsPerSlotInLds>(a, 5, row_groups);  // 8 * 2 * 8 KiB of rows
 }
 
-template <int BS, bool HAS_ZP>
+template <int BS, bool HAS_ZP, bool ROW>
 int launch_shape(const blkq4_gemm_args* a) {
   if (a->m > 16) {
     // Every workgroup fetches the 32 rows of its group for all of K, so wide workgroups (more column tiles)
@@ -363,27 +413,39 @@ int launch_shape(const blkq4_gemm_args* a) {
     constexpr int kComputeUnits = 256;
     const int row_groups = (a->m + 31) / 32;
     const long tiles = static_cast<long>(a->n / 16) * row_groups;
-    if (tiles >= 4 * kComputeUnits) return launch_rows<BS, HAS_ZP, 4>(a, row_groups);
-    if (tiles >= 2 * kComputeUnits) return launch_rows<BS, HAS_ZP, 2>(a, row_groups);
-    return launch_rows<BS, HAS_ZP, 1>(a, row_groups);
+    if (tiles >= 4 * kComputeUnits) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 4>(a, row_groups);
+    if (tiles >= 2 * kComputeUnits) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 2>(a, row_groups);
+    return launch_rows<BS, HAS_ZP, ROW, 1>(a, row_groups);
   }
   int nt, depth;
   choose_shape(a->m, a->n, &nt, &depth);
-  if (nt == 1 && depth == 8) return launch_waves<BS, HAS_ZP, 8, 1>(a);
-  if (nt == 1) return launch_waves<BS, HAS_ZP, 4, 1>(a);
-  if (nt == 2) return launch_waves<BS, HAS_ZP, 4, 2>(a);
-  return launch_waves<BS, HAS_ZP, 4, 3>(a);
+  if (ROW) {
+    // blocks along N: 28 registers of packed weights, scales and zero-points per slot and tile, so one tile
+    return (depth == 8) ? launch_waves<BS, HAS_ZP, ROW, 8, 1>(a) : launch_waves<BS, HAS_ZP, ROW, 4, 1>(a);
+  }
+  if (nt == 1 && depth == 8) return launch_waves<BS, HAS_ZP, ROW, 8, 1>(a);
+  if (nt == 1) return launch_waves<BS, HAS_ZP, ROW, 4, 1>(a);
+  if (nt == 2) return launch_waves<BS, HAS_ZP, ROW, 4, ROW ? 1 : 2>(a);
+  return launch_waves<BS, HAS_ZP, ROW, 4, ROW ? 1 : 3>(a);
 }
 
 template <int BS>
 int launch_skinny(const blkq4_gemm_args* a) {
-  return a->zero_points ? launch_shape<BS, true>(a) : launch_shape<BS, false>(a);
+  if (a->column_wise) return a->zero_points ? launch_shape<BS, true, false>(a) : launch_shape<BS, false, false>(a);
+  return a->zero_points ? launch_shape<BS, true, true>(a) : launch_shape<BS, false, true>(a);
 }
 
 }  // namespace
 
 extern "C" int blkq4_dev_skinny(const blkq4_gemm_args* a) {
   if (a->m < 1 || a->m > kStreamingMaxRows || (a->n % 16) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
+  if (!a->column_wise) {
+    // blocks along N: a 16-column tile lies inside one block, and the meta data are fetched 16 bytes at a time
+    if ((a->n % a->block_size) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 15u) != 0 ||
+        (reinterpret_cast<uintptr_t>(a->zero_points) & 15u) != 0) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+  }
   switch (a->block_size) {
     case 16: return launch_skinny<16>(a);
     case 32: return launch_skinny<32>(a);
