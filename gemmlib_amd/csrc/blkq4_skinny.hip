@@ -1,24 +1,30 @@
-// M = 1..16 path (decode GEMV and small-batch GEMM) for gfx950.
+// Weight-streaming kernel for gfx950: decode GEMV, small-batch GEMM and, in row groups of 32, every M
+// for which streaming the weights once per row group beats the tile kernel.
 //
 // The work is a stream over the packed weights (K*N/2 bytes plus scales and zero-points) that has to
 // run at HBM speed; everything else is arranged so that the stream is requested as early and as
 // deeply as possible and nothing serialises behind it:
-//   - a workgroup of four or eight waves owns 16, 32 or 48 output columns and the whole K range; the waves split K in
-//     128-deep slices, so every wave load is one 16-byte unit per lane: 16 columns x 4 consecutive
-//     k-units = four contiguous 256-byte runs of the packed layout;
-//   - a wave keeps the weight units, scales and zero-points of kDepth slices in flight and refills a
+//   - a workgroup of 4, 8 or 16 waves owns 16 * NT output columns, 16 * MT rows and the whole K range; the
+//     waves split K in 128-deep slices, so every wave load is one 16-byte unit per lane: 16 columns x 4
+//     consecutive k-units = four contiguous 256-byte runs of the packed layout;
+//   - a wave keeps the weight units, scales and zero-points of DEPTH slices in flight and refills a
 //     slot as soon as it has consumed it (out-of-range slices wrap around to valid units and are
 //     multiplied by a zero scale, so the loop has no divergent loads);
-//   - the activation rows (at most 16 x K fp16) are copied once per workgroup into LDS by asynchronous
-//     global_load_lds copies issued before the first weight request, laid out per 32-deep unit as
-//     [unit][row][64 bytes] (16-byte chunks XOR-swizzled with bits 2..3 of the row so that a fragment
-//     read is free of bank conflicts); when they do not fit (K too large) the lanes that carry a row
-//     load their 64 bytes per slice straight from global memory (L2 resident) into the same ring;
-//   - a lane multiplies its (column, 32 k) of weights with the matching 32 k of up to 16 activation
-//     rows through v_mfma_f32_16x16x32_f16 (weights as the row operand: a lane ends up with 4
-//     consecutive output columns of one activation row, one 8-byte store);
-//   - the waves' partial tiles are summed through LDS by wave 0: no atomics, no scratch buffer.
-// Dequantization happens in registers (blkq4_dequant.h); accumulation is fp32.
+//   - the activation rows are copied into LDS by asynchronous global_load_lds copies, laid out per 32-deep
+//     unit as [unit][row][64 bytes] (16-byte chunks XOR-swizzled with bits 2..3 of the row so that a
+//     fragment read is free of bank conflicts): once per workgroup, before the first weight request, when
+//     all of K fits; otherwise per slot, private to the wave and requested right before the slot's
+//     weights, so that a wave that has its weights has its rows and no barrier is needed;
+//   - a lane dequantizes its (column, 32 k) of weights once and multiplies them with the matching 32 k of
+//     MT tiles of 16 activation rows through v_mfma_f32_16x16x32_f16 (weights as the row operand: a lane
+//     ends up with 4 consecutive output columns of one activation row per tile);
+//   - the waves' partial tiles are summed through LDS (the space of the activation rows, once every wave
+//     is done with them) by all threads: no atomics, no scratch buffer;
+//   - more than 32 rows: the grid has one workgroup per (row group of 32, column group); the row groups
+//     of a column group run on the same XCD, so the weights they share are fetched into its L2 once.
+// Dequantization happens in registers (blkq4_dequant.h), for blocks along K (a scale per column and block
+// row) and along N (a scale per k, shared by BS columns, in the reference's packed order); accumulation
+// is fp32.
 
 #include <hip/hip_runtime.h>
 
@@ -32,9 +38,7 @@ namespace {
 
 using namespace blkq4;
 
-
 // Where a wave finds its activation fragments.
-constexpr int kRowsInRegisters = 0;  // each lane loads its rows' 64 bytes per slice into the ring of slots
 constexpr int kRowsWholeInLds = 1;   // all rows, all of K, staged once per workgroup
 constexpr int kRowsPerSlotInLds = 2; // 16 * MT rows x 128 k staged per slot, private to the wave
 
@@ -48,7 +52,6 @@ struct Slot {
   // the meta data (two 16-row groups of 32 + 16 bytes)
   uint4 rs[ROW ? NT : 1][4];
   uint4 rz[ROW ? NT : 1][2];
-  uint4 a[AM == kRowsInRegisters ? 4 * MT : 1];  // 32 k of this lane's activation rows (unused when they are in LDS)
 };
 
 // kWaves: waves of the workgroup, which split K.  DEPTH: k slices (128 deep) a wave keeps in flight.  NT: 16-column tiles per wave that share one
@@ -104,14 +107,6 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     n[t] = ((tile < tiles) ? tile : cg * NT) * 16 + nl;
   }
   const DequantMasks masks = DequantMasks::make();
-  // lanes without a row (past M) re-read the last row: an output element depends on its own activation
-  // row only, and the rows past M are never stored
-  const uint8_t* a_row[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    a_row[mt] = reinterpret_cast<const uint8_t*>(A) + static_cast<size_t>(min(16 * mt + nl, M - 1)) * K * 2;
-  }
-
   const int units = K >> 5;             // 32-deep units
   const int slices = (units + 3) >> 2;  // 128-deep slices (the last one may be half full)
   const int my_slices = (slices - wave + kWaves - 1) / kWaves;  // slices wave, wave + kWaves, ...
@@ -196,14 +191,6 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
         }                                                                                      \
       }                                                                                        \
     }                                                                                          \
-    if (AM == kRowsInRegisters) {                                                              \
-      _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                      \
-        const uint4* p_ = reinterpret_cast<const uint4*>(a_row[mt] + static_cast<size_t>(ksg_) * 64); \
-        _Pragma("unroll") for (int j = 0; j < (AM == kRowsInRegisters ? 4 : 0); ++j) {         \
-          (dst_).a[(AM == kRowsInRegisters) ? 4 * mt + j : 0] = p_[j];                         \
-        }                                                                                      \
-      }                                                                                        \
-    }                                                                                          \
   }
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) BLKQ4_LOAD_SLOT(slot[d], d, wave + d * kWaves);
@@ -229,7 +216,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
           for (int j = 0; j < 4; ++j) {
             af[mt][j] = as_half8(*reinterpret_cast<const uint4*>(ap + mt * 1024 + ((j ^ a_swz) * 16)));
           }
-      } else if (AM == kRowsPerSlotInLds) {
+      } else {
         // the rows of this slot were requested before its weights; younger than them are those weights and
         // everything the other DEPTH - 1 slots have requested since
         constexpr int kYounger = kLoads + (DEPTH - 1) * (4 * MT + kLoads);
@@ -241,11 +228,6 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
           for (int j = 0; j < 4; ++j) {
             af[mt][j] = as_half8(*reinterpret_cast<const uint4*>(ap + mt * 1024 + ((j ^ a_swz) * 16)));
           }
-      } else {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) af[mt][j] = as_half8(slot[d].a[(AM == kRowsInRegisters) ? 4 * mt + j : 0]);
       }
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
@@ -301,7 +283,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 #undef BLKQ4_LOAD_SLOT
 
   // cross-wave reduction through LDS (which holds activation rows until every wave is done with them)
-  if (AM != kRowsInRegisters) __syncthreads();
+  __syncthreads();
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
