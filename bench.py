@@ -228,6 +228,62 @@ def bench_copy(torch, capi, device, steps, warmup):
     }
 
 
+def bench_context(torch, capi, device, head_problem, steps, warmup):
+    """Figures the headline numbers are read against, measured in the same run:
+    * what a graph node costs when its kernel does nothing, and what a kernel costs that issues the GEMV's
+      memory requests and nothing else (the probe library built next to the product library);
+    * the vendor library's plain fp16 GEMM (torch.matmul on an fp16 copy of the dequantized-size weight
+      matrix, no 4-bit weights involved) on the headline shape;
+    * the headline GEMM on all-zero activations and weights: same instruction stream, idle data paths --
+      the difference to the real run is what the clock loses under load."""
+    import ctypes
+    from gemmlib_amd import build as _build
+    out = {}
+    probe = ctypes.CDLL(_build.PROBE_PATH)
+    probe.blkq4_probe_empty.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    probe.blkq4_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                         ctypes.c_void_p, ctypes.c_void_p]
+    scratch = torch.zeros(1 << 16, dtype=torch.int32, device=device)
+
+    def stream_ptr():
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    wall, evt, _ = timed_region(torch, [lambda: probe.blkq4_probe_empty(scratch.data_ptr(), stream_ptr())], steps, warmup)
+    out["empty_kernel_us"] = round(evt / steps * 1e6, 3)
+    m, k, n, bs, has_offsets, _ = CONFIGS["C2"]
+    per_set = k * n // 2 + 2 * k * n // bs
+    copies = INFINITY_CACHE_BYTES // per_set + 2
+    ws = [torch.randint(0, 256, (k * n // 2,), dtype=torch.uint8, device=device) for _ in range(copies)]
+    ss = [torch.ones(k // bs * n, dtype=torch.float16, device=device) for _ in range(copies)]
+    for with_scales in (False, True):
+        launches = [(lambda w=w, sc=sc: probe.blkq4_probe_stream(w.data_ptr(), sc.data_ptr() if with_scales else None,
+                                                                 n, k, scratch.data_ptr(), stream_ptr()))
+                    for w, sc in zip(ws, ss)]
+        wall, evt, _ = timed_region(torch, launches, steps, warmup)
+        out["c2_requests_only_us" if with_scales else "c2_weight_requests_only_us"] = round(evt / steps * 1e6, 3)
+    del ws, ss
+    if head_problem is not None:
+        a, sets, c, w_host = head_problem
+        m, k, n, bs, has_offsets, _ = CONFIGS["C4"]
+        b = (torch.randn(n, k, device=device, dtype=torch.float32) * 0.02).to(torch.float16).t()
+        wall, evt, _ = timed_region(torch, [lambda: torch.matmul(a, b)], steps, warmup)
+        out["library_fp16_gemm_c4_shape"] = {"us": round(evt / steps * 1e6, 3),
+                                             "tflops": round(2.0 * m * n * k / (evt / steps) / 1e12, 3)}
+        del b
+        m5, k5, n5 = CONFIGS["C5"][:3]
+        a5 = torch.randn(m5, k5, device=device, dtype=torch.float32).to(torch.float16)
+        b5 = (torch.randn(n5, k5, device=device, dtype=torch.float16) * 0.02).t()
+        wall, evt, _ = timed_region(torch, [lambda: torch.matmul(a5, b5)], max(10, steps // 10), max(2, warmup // 10))
+        per = evt / max(10, steps // 10)
+        out["library_fp16_gemm_c5_shape"] = {"us": round(per * 1e6, 3), "tflops": round(2.0 * m5 * n5 * k5 / per / 1e12, 3)}
+        del a5, b5
+        q_w, q_s, q_zp = sets[0]
+        za, zw, zs, zz = torch.zeros_like(a), torch.zeros_like(q_w), torch.zeros_like(q_s), torch.zeros_like(q_zp)
+        wall, evt, _ = timed_region(torch, [lambda: capi.gemm(bs, True, m, n, k, za, zw, zs, zz, c)], steps, warmup)
+        out["c4_all_zero_data_us"] = round(evt / steps * 1e6, 3)
+    return out
+
+
 def cpu_baseline(name, a_dev, w_host, target_seconds=12.0):
     """The oracle's dequantize + GEMM on a bounded sample of rows of the same workload."""
     import numpy as np
@@ -266,6 +322,7 @@ def main(argv=None) -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-context", action="store_true", help="skip the floors and the library comparison")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -310,6 +367,8 @@ def main(argv=None) -> int:
     if "C2" in results:
         line["gemv"] = {"workload": results["C2"]["workload"], "value": results["C2"]["value"], "unit": "GB/s",
                         "kernel_us": results["C2"]["kernel_us"], "roofline": results["C2"]["roofline"]}
+    if not args.no_context:
+        line["context"] = bench_context(torch, capi, device, head_problem, args.steps, args.warmup)
     if not args.no_cpu and head_problem is not None:
         a, sets, out, w_host = head_problem
         line["cpu_baseline"] = cpu_baseline("C4", a, w_host)

@@ -23,6 +23,7 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 OBJ_DIR = os.path.join(PKG_DIR, "build")
 INCLUDE = os.path.join(ROOT, "include")
 LIB_PATH = os.path.join(LIB_DIR, "libms_blkq4gemm.so")
+PROBE_PATH = os.path.join(LIB_DIR, "libblkq4_probe.so")  # measurement aids for bench.py, not part of the product
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -70,6 +71,7 @@ def build_library(verbose: bool = True) -> str:
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
         list(pool.map(lambda j: _run(*j), jobs))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs], "packed-fp32-ops")
+    _run([HIPCC, *HIP_FLAGS, "-shared", "-o", PROBE_PATH, os.path.join(CSRC, "blkq4_probe.hip")], "packed-fp32-ops")
     if verbose:
         print(f"built {LIB_PATH}")
     return LIB_PATH
