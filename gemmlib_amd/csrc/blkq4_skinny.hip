@@ -80,13 +80,16 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   const uint8_t* a_lds = smem;
 
   // Workgroup -> (row group of 16 * MT rows, group of NT column tiles).  Consecutive workgroups go to
-  // consecutive XCDs; the row groups of one column group are 8 apart, so they run on the same XCD and the
-  // weights they share stay in that XCD's L2.
+  // consecutive XCDs (8 of them).  An XCD's workgroups take, in this order: the row groups of a column
+  // group (they share its weights), then the next of four neighbouring column groups (they share the 128-byte
+  // lines of the scale and zero-point rows, and their weights are contiguous), so that what is shared is
+  // fetched into that XCD's L2 once.
   const int col_groups = ((N >> 4) + NT - 1) / NT;
   const int wg = blockIdx.x;
-  const int rg = (wg >> 3) % row_groups;
-  const int cg = (wg & 7) + 8 * ((wg >> 3) / row_groups);
-  if (cg >= col_groups) return;  // the grid is rounded up to whole groups of 8
+  const int q = wg >> 3;
+  const int rg = q % row_groups;
+  const int cg = 4 * ((wg & 7) + 8 * ((q / row_groups) >> 2)) + ((q / row_groups) & 3);
+  if (cg >= col_groups) return;  // the grid is rounded up to whole groups of 32 column groups
   const int m0 = rg * (16 * MT);
   const int M = min(16 * MT, M_total - m0);
   A += static_cast<size_t>(m0) * K;
@@ -351,7 +354,7 @@ int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
   if (attr != hipSuccess) return static_cast<int>(attr);
   const int col_groups = (a->n / 16 + NT - 1) / NT;
-  const unsigned grid = static_cast<unsigned>((col_groups + 7) / 8) * 8u * static_cast<unsigned>(row_groups);
+  const unsigned grid = static_cast<unsigned>((col_groups + 31) / 32) * 32u * static_cast<unsigned>(row_groups);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * kWaves), lds_bytes, static_cast<hipStream_t>(a->stream),
                      static_cast<const uint16_t*>(a->a), static_cast<const uint4*>(a->packed_w),
                      static_cast<const uint16_t*>(a->scales), static_cast<const uint8_t*>(a->zero_points),
