@@ -36,8 +36,10 @@ CONFIGS = {
     "C4": (2048, 4096, 4096, 64, True, "mfma"),
     "C5": (4096, 8192, 28672, 16, True, "mfma"),
     "C4r": (2048, 4096, 4096, 64, True, "mfma"),
+    "C2r": (1, 4096, 4096, 64, False, "hbm"),
+    "M128": (128, 4096, 4096, 64, True, "hbm"),
 }
-COLUMN_WISE = {"C4r": False}
+COLUMN_WISE = {"C4r": False, "C2r": False}
 DESCRIPTION = {
     "C1": "C1 CPU-runnable case M=64 K=1024 N=1024 bs32 asym",
     "C2": "C2 decode GEMV M=1 K=4096 N=4096 bs64 sym",
@@ -45,6 +47,8 @@ DESCRIPTION = {
     "C4": "C4 prefill GEMM M=2048 K=4096 N=4096 bs64 asym",
     "C5": "C5 large-layer GEMM M=4096 K=8192 N=28672 bs16 asym",
     "C4r": "C4 shape with blocks along N (column_wise_blocking=false) M=2048 K=4096 N=4096 bs64 asym",
+    "C2r": "C2 shape with blocks along N (column_wise_blocking=false) M=1 K=4096 N=4096 bs64 sym",
+    "M128": "mid-size batch M=128 K=4096 N=4096 bs64 asym (streaming kernel in four row groups)",
 }
 
 
@@ -320,7 +324,7 @@ def main(argv=None) -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r")
+    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r,C2r,M128")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-context", action="store_true", help="skip the floors and the library comparison")
     args = ap.parse_args(argv)
