@@ -27,11 +27,12 @@ inline void set_error(std::string* err, std::string&& text) {
 // round of 256 workgroups, 0.64 us a step with 128 x 256 tiles and 0.42 us with the 128 x 128 tiles it uses
 // when those cover the problem in one round.
 inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k) {
-  if (!column_wise) return m <= 384;  // blocks along N: the tile kernel for them is a plain one (K=N=4096: 99 us at m = 256)
   if (m <= 32) return true;
   if (m > 1024) return false;
   const double row_groups = (m + 31) / 32;
-  const double streaming_us = 2.8 * row_groups * (static_cast<double>(n) / 4096.0) * (static_cast<double>(k) / 4096.0);
+  // blocks along N: the streaming kernel converts with 23 instead of 13 instructions per 8 weights
+  const double streaming_us = (column_wise ? 2.8 : 5.6) * row_groups * (static_cast<double>(n) / 4096.0) *
+                              (static_cast<double>(k) / 4096.0);
   const long small_tiles = static_cast<long>((m + 127) / 128) * ((n + 127) / 128);
   const long workgroups = static_cast<long>((m + 127) / 128) * ((n + 255) / 256);
   const double tile_us = (small_tiles <= 256) ? (k / 64) * 0.42
@@ -231,7 +232,7 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
     set_error(err, "Kernel execution failed: Error Misaligned Operand");
     return -1;
   }
-  // blocks along N: the kernel fetches scales and zero-points 16 bytes at a time
+  // blocks along N: the streaming kernel fetches scales and zero-points 16 bytes at a time
   if (!column_wise_blocking && (!aligned16(scales_ptr) || (has_offsets && !aligned16(offsets_ptr)))) {
     set_error(err, "Kernel execution failed: Error Misaligned Operand");
     return -1;
@@ -254,9 +255,7 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
   args.c = output_ptr;
   args.stream = stream;
   // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
-  const int code = streaming_kernel_takes(column_wise_blocking, m, n, k) ? blkq4_dev_skinny(&args)
-                   : column_wise_blocking                                ? blkq4_dev_gemm(&args)
-                                                                         : blkq4_dev_gemm_rowwise(&args);
+  const int code = streaming_kernel_takes(column_wise_blocking, m, n, k) ? blkq4_dev_skinny(&args) : blkq4_dev_gemm(&args);
   if (code) return device_failure(code, err);
   return 0;
 }

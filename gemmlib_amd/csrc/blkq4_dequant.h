@@ -88,6 +88,30 @@ __device__ __forceinline__ half2_t dequant_pair(uint32_t w_shifted, int pair, co
   return (as_half2((w_shifted & m.hi_mask) | m.magic_64) + c.neg_c1) * c.scale2;
 }
 
+// Blocks along N: the constants that one pair of weights is added to, built from the packed zero-point
+// word of the pair (reference order: bytes 0 and 2 of the word are rows 2p and 2p + 1 of the 16-row group,
+// bytes 1 and 3 rows 2p + 8 and 2p + 9).  hh selects the rows (0: the first eight of the group), pair
+// parity the magic number (even pairs 1024 + q, odd pairs 64 + q with the zero-point shifted likewise).
+struct RowMetaMasks {
+  uint32_t byte_pair, byte_pair_x16, neg_1024, neg_64;
+  __device__ __forceinline__ static RowMetaMasks make() {
+    RowMetaMasks m;
+    m.byte_pair = DequantMasks::opaque(0x00ff00ffu);
+    m.byte_pair_x16 = DequantMasks::opaque(0x0ff00ff0u);
+    m.neg_1024 = DequantMasks::opaque(0xE400E400u);
+    m.neg_64 = DequantMasks::opaque(0xD400D400u);
+    return m;
+  }
+};
+template <bool HAS_ZP>
+__device__ __forceinline__ half2_t row_neg_c(uint32_t zp_word, int pair, int hh, const RowMetaMasks& m) {
+  if (!HAS_ZP) return as_half2((pair & 1) == 0 ? 0xE408E408u : 0xD480D480u);  // zero-point 8
+  if ((pair & 1) == 0) return as_half2((((hh == 0) ? zp_word : (zp_word >> 8)) & m.byte_pair) | m.neg_1024);
+  return as_half2((((hh == 0) ? (zp_word << 4) : (zp_word >> 4)) & m.byte_pair_x16) | m.neg_64);
+}
+// component c of a 4-word vector, c known at compile time after unrolling
+__device__ __forceinline__ uint32_t vec_word(const uint4& v, int c) { return c == 0 ? v.x : c == 1 ? v.y : c == 2 ? v.z : v.w; }
+
 __device__ __forceinline__ half8_t as_half8(uint4 v) {
   uint4_t t = {v.x, v.y, v.z, v.w};
   return __builtin_bit_cast(half8_t, t);

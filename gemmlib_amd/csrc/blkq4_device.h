@@ -67,9 +67,8 @@ typedef struct {
 } blkq4_repack_args;
 
 int blkq4_dev_prepack(const blkq4_prepack_args* args);
-int blkq4_dev_gemm(const blkq4_gemm_args* args);   /* m > 16: MFMA tile kernel */
-int blkq4_dev_skinny(const blkq4_gemm_args* args); /* 1 <= m <= 16 */
-int blkq4_dev_gemm_rowwise(const blkq4_gemm_args* args); /* column_wise = 0, every m */
+int blkq4_dev_gemm(const blkq4_gemm_args* args);   /* MFMA tile kernel, every m (made for large m) */
+int blkq4_dev_skinny(const blkq4_gemm_args* args); /* weight-streaming kernel, 1 <= m <= 1024 */
 int blkq4_dev_repack(const blkq4_repack_args* args);
 const char* blkq4_dev_error_string(int code);
 

@@ -1,10 +1,11 @@
-// M > 16 path: fp16 MFMA GEMM with the 4-bit weights dequantized in registers (gfx950).
+// Tile kernel: fp16 MFMA GEMM with the 4-bit weights dequantized in registers (gfx950), for the row
+// counts the weight-streaming kernel does not take.
 //
-// Workgroup tile (32*RT) x 128 x 64 (M x N x K), four waves side by side along N: a wave owns
-// (32*RT) x 32 outputs, i.e. ONE 32-column weight fragment per 16-deep k step that it converts to
-// fp16 once and feeds to RT MFMAs (RT = 8 for large M).  Measured on MI355X, a wave can issue about
-// four VALU instructions in the shadow of one 32x32x16 MFMA; the tall wave tile keeps the
-// conversion at 13 VALU instructions per 8 MFMAs.
+// A workgroup is WM x WN computing waves, each owning (32*RT) x (32*NT) outputs, plus PW producer waves
+// that only issue copies (see launch_rt for the shapes in use: 256 x 256, 128 x 256 and 128 x 128 tiles).
+// A wave converts each of its NT 32-column weight fragments to fp16 once per 16-deep k step and feeds it
+// to RT MFMAs; a wave can issue about five VALU instructions in the shadow of one 32x32x16 MFMA, and the
+// conversion takes 13 per fragment and step.
 //
 // Data movement: everything the main loop consumes is copied HBM -> LDS by the asynchronous
 // global_load_lds_dwordx4 / _dword instructions (no registers in between) into a ring of kStages
@@ -17,21 +18,26 @@
 //   - packed weights: a lane's MFMA operand for one 64-deep k tile is exactly one 16-byte unit of
 //     the packed layout (32 consecutive k of one column); 32 lanes request 512 contiguous bytes and
 //     every lane later reads back the unit it requested;
-//   - scales (and zero-points) of the tile: one 4-byte request per lane and quantization block row.
+//   - scales (and zero-points) of the tile: blocks along K, one 4-byte request per lane and
+//     quantization block row; blocks along N (ROW), the 128 + 64 bytes per column group as they lie in
+//     memory (the reference's packed order is made for packed fp16 arithmetic and is used as it is).
 //
-// Schedule of one k tile (four 16-deep steps, RT MFMAs each), written out in program order and
+// Schedule of one k tile (four 16-deep steps, RT*NT MFMAs each), written out in program order and
 // pinned with scheduling barriers because the compiler's own schedule serialises LDS latency:
-//   after MFMA r of step j come the LDS read of activation fragment r of step j+1 and one piece
-//   (3-4 VALU instructions) of the next weight fragment's conversion, so that the issue slots in the
+//   behind every MFMA come the LDS read of an activation fragment of step j+1 and one stage of the
+//   conversion of two pieces of the next weight fragments (two pieces interleaved: a packed instruction
+//   that reads the result of the one before it costs a wait state), so that the issue slots in the
 //   shadow of every MFMA are filled and nothing is consumed sooner than one step after its request.
 //   After step 1 one s_waitcnt vmcnt + s_barrier publish the NEXT k tile, so that steps 2 and 3 can
 //   already read its packed weights / scales and the fragments of its step 0: the MFMA pipe never
 //   waits for the first LDS read of a tile.  The asynchronous copies for the tile kDistance ahead
-//   are issued one per MFMA in steps 2 and 3 (a copy instruction can stall at issue while the
-//   texture path drains; behind an MFMA that stall is hidden).
+//   are spread over the MFMAs of the steps after the barrier that frees their ring slot (a copy
+//   instruction can stall at issue while the texture path drains; behind an MFMA that stall is hidden),
+//   or left to the producer waves.
 //
 // Math: v_mfma_f32_32x32x16_f16 with the weights as the row operand, so the accumulator of a lane
-// holds 4 consecutive output columns of one activation row (8-byte stores in the epilogue).
+// holds 4 consecutive output columns of one activation row; the epilogue transposes the tile through
+// LDS and stores whole rows.
 //
 // Rows past M and 32-column tiles past N are handled by clamping the addresses that are read (the
 // values computed from them are never stored), so the main loop has no branches.
@@ -66,31 +72,42 @@ constexpr int stage_slot(int g, int u, int pairs, int slots) {
 // Shape of a workgroup: WM x WN waves, each owning (32*RT) rows x (32*NT) columns (the WM waves of a
 // column group share its packed weights, scales and zero-points), plus PW producer waves that do
 // nothing but issue the async copies.  With PW = 0 the computing waves issue the copies themselves.
-template <int BS, int RT, int NT, int WM, int WN, int PW>
+// ROW: quantization blocks run along N (one k, BS columns).  The scales and zero-points of a k tile are
+// then, per group of BS columns, 64 consecutive rows in the packed order described in blkq4_device.h:
+// 128 + 64 bytes, copied as they are.
+template <int BS, int RT, int NT, int WM, int WN, int PW, bool ROW>
 struct Stage {
   static constexpr int kCopiers = (PW > 0) ? PW : WM * WN;     // waves that share out the copies of a stage
   static constexpr int kBlocks = kBK / BS;                     // quantization block rows per k tile
   static constexpr int kABytes = 32 * RT * WM * 128;           // [row][8 x 16-byte units, swizzled]
   static constexpr int kBBytes = WN * NT * 1024;               // [column group][fragment][lane] 16-byte units
-  static constexpr int kMetaBytes = WN * kBlocks * 256;        // [column group][block][2 fragments][64 B scales | 32 B zps | pad]
+  // blocks along K: [column group][block][2 fragments][64 B scales | 32 B zps | pad]
+  // blocks along N: [group of BS columns][128 B scales], then [group][64 B zero-points] (at least 256 B:
+  // one copy instruction writes 256 B)
+  static constexpr int kGroups = 32 * NT * WN / BS;            // column groups of a workgroup tile (ROW)
+  static constexpr int kRowScaleOps = kGroups / 2;             // copies of 2 x 128 B
+  static constexpr int kRowZpOps = (kGroups + 3) / 4;          // copies of 4 x 64 B
+  static constexpr int kMetaBytes = ROW ? kGroups * 128 + kRowZpOps * 256 : WN * kBlocks * 256;
   static constexpr int kBytes = kABytes + kBBytes + kMetaBytes;
   // per copying wave and stage: 8-row activation groups, packed weight fragments, scale / zero-point rows
   static constexpr int kAOps = (4 * RT * WM + kCopiers - 1) / kCopiers;
   static constexpr int kBOps = (NT * WN + kCopiers - 1) / kCopiers;
-  static constexpr int kMOps = (WN * kBlocks + kCopiers - 1) / kCopiers;
+  static constexpr int kMTotal = ROW ? kRowScaleOps + kRowZpOps : WN * kBlocks;
+  static constexpr int kMOps = (kMTotal + kCopiers - 1) / kCopiers;
   static constexpr int kOps = kAOps + kBOps + kMOps;
   // ring of k tiles in LDS, requested kDistance tiles ahead of the one being consumed
   static constexpr int kStages = (4 * kBytes <= 160 * 1024) ? 4 : 3;
   static constexpr int kDistance = kStages - 1;  // the slot being refilled is the one nobody reads
 };
 
-template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW>
+template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW>
 __global__ __launch_bounds__(64 * (WM * WN + PW))
     __attribute__((amdgpu_waves_per_eu((WM * WN + PW) / 4, (WM * WN + PW) / 4))) void gemm_mfma_kernel(
         const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ S,
         const uint8_t* __restrict__ Z, uint16_t* __restrict__ C, int M, int N, int K, int m_tiles) {
-  using St = Stage<BS, RT, NT, WM, WN, PW>;
+  using St = Stage<BS, RT, NT, WM, WN, PW, ROW>;
   constexpr int kComputeWaves = WM * WN;
+  static_assert(!ROW || St::kGroups % 2 == 0, "scale copies take two column groups at a time");
   constexpr int kCopiers = St::kCopiers;
   static_assert((WM * WN + PW) % 4 == 0, "whole waves per SIMD");
   constexpr int kBlocks = St::kBlocks;
@@ -151,22 +168,45 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
     b_dst[p] = St::kABytes + f * 1024;
   }
   const uint32_t b_stride = static_cast<uint32_t>(N) * 32u;  // two 32-deep units per k tile
-  // meta: one copy per (column group, block row).  Per 32-lane half (= fragment): lanes 0..15 fetch 2
-  // scales each, lanes 16..23 fetch 4 zero-points each.  The copy lands at 4 * lane inside a 256-byte
-  // row, so the lanes with nothing to fetch write into padding; they re-read a scale so that the copy
-  // needs no branch.
+  // meta, blocks along K: one copy per (column group, block row).  Per 32-lane half (= fragment): lanes
+  // 0..15 fetch 2 scales each, lanes 16..23 fetch 4 zero-points each.  The copy lands at 4 * lane inside a
+  // 256-byte row, so the lanes with nothing to fetch write into padding; they re-read a scale so that the
+  // copy needs no branch.
+  // meta, blocks along N: the 128 bytes of scales of two column groups per copy (32 lanes each), then the
+  // 64 bytes of zero-points of four column groups per copy (16 lanes each); a group past N re-reads the
+  // last one.
   constexpr int kMOps = St::kMOps;
   const bool meta_is_scale = i < 16 || i >= 24 || !HAS_ZP;
   const uint32_t meta_row_bytes = meta_is_scale ? static_cast<uint32_t>(N) * 2u : static_cast<uint32_t>(N);
   const uint8_t* meta_ptr[kMOps];
   uint32_t meta_dst[kMOps];
+  uint32_t meta_step[kMOps];  // bytes from one k tile to the next
 #pragma unroll
   for (int p = 0; p < kMOps; ++p) {
-    const int idx = (kCopiers * p + cw) % (WN * kBlocks);  // column group idx / kBlocks, block row idx % kBlocks
-    const int nb = min(bn * kBN + (idx / kBlocks) * (32 * NT) + ((NT == 2) ? 32 * h : 0), N - 32);
-    meta_ptr[p] = (meta_is_scale ? S + static_cast<size_t>(nb + 2 * (i & 15)) * 2 : Z + (nb + 4 * (i & 7))) +
-                  static_cast<size_t>(idx % kBlocks) * meta_row_bytes;
-    meta_dst[p] = St::kABytes + St::kBBytes + idx * 256;
+    const int idx = (kCopiers * p + cw) % St::kMTotal;
+    if (ROW) {
+      const int last_group = N / BS - 1;
+      const int group0 = bn * kBN / BS;
+      if (idx < St::kRowScaleOps) {
+        const int grp = min(group0 + 2 * idx + (lane >> 5), last_group);
+        meta_ptr[p] = S + (static_cast<size_t>(grp) * K) * 2 + (lane & 31) * 4;
+        meta_dst[p] = St::kABytes + St::kBBytes + idx * 256;
+        meta_step[p] = 128;
+      } else {
+        const int z = idx - St::kRowScaleOps;
+        const int grp = min(group0 + min(4 * z + (lane >> 4), St::kGroups - 1), last_group);
+        meta_ptr[p] = (HAS_ZP ? Z + static_cast<size_t>(grp) * K : S) + (lane & 15) * 4;
+        meta_dst[p] = St::kABytes + St::kBBytes + St::kGroups * 128 + z * 256;
+        meta_step[p] = 64;
+      }
+    } else {
+      // column group idx / kBlocks, block row idx % kBlocks
+      const int nb = min(bn * kBN + (idx / kBlocks) * (32 * NT) + ((NT == 2) ? 32 * h : 0), N - 32);
+      meta_ptr[p] = (meta_is_scale ? S + static_cast<size_t>(nb + 2 * (i & 15)) * 2 : Z + (nb + 4 * (i & 7))) +
+                    static_cast<size_t>(idx % kBlocks) * meta_row_bytes;
+      meta_dst[p] = St::kABytes + St::kBBytes + idx * 256;
+      meta_step[p] = kBlocks * meta_row_bytes;
+    }
   }
 
   const uint32_t lds0 = static_cast<uint32_t>(
@@ -186,8 +226,7 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
       async_copy_16(sbase_ + b_dst[p_], W + static_cast<size_t>(tile_) * b_stride, b_off[p_]);            \
     } else {                                                                                              \
       const int p_ = ((q_) >= kAOps + kBOps) ? (q_) - kAOps - kBOps : 0;                                   \
-      async_copy_4_flat(sbase_ + meta_dst[p_],                                                            \
-                        meta_ptr[p_] + static_cast<size_t>(tile_) * (kBlocks * meta_row_bytes));           \
+      async_copy_4_flat(sbase_ + meta_dst[p_], meta_ptr[p_] + static_cast<size_t>(tile_) * meta_step[p_]); \
     }                                                                                                     \
   }
 
@@ -251,8 +290,17 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   }
   const uint32_t b_rd = lds0 + St::kABytes + wn * (NT * 1024) + lane * 16;
   const uint32_t m_rd = lds0 + St::kABytes + St::kBBytes + wn * kBlocks * 256;
+  // blocks along N: the 16-row groups 2h and 2h + 1 of the column group of this lane's column, per fragment
+  uint32_t msc_rd[NT], mzp_rd[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int gl = (wn * (32 * NT) + 32 * t + i) / BS;
+    msc_rd[t] = lds0 + St::kABytes + St::kBBytes + gl * 128 + h * 64;
+    mzp_rd[t] = lds0 + St::kABytes + St::kBBytes + St::kGroups * 128 + gl * 64 + h * 32;
+  }
 
   const DequantMasks masks = DequantMasks::make();
+  const RowMetaMasks rmasks = RowMetaMasks::make();
 
 #define BLKQ4_READ_A1(dst_, stage_off_, j_, r_) (dst_)[r_] = as_half8(lds_read_16((stage_off_) + a_rd[j_], (r_) * 4096))
   // packed words, scales and zero-points of all the wave's fragments for one k tile
@@ -263,16 +311,33 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
     (words_)[t][1] = u_.y;                                                                   \
     (words_)[t][2] = u_.z;                                                                   \
     (words_)[t][3] = u_.w;                                                                   \
-    _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                      \
-      const int blk_ = (BS == 64) ? 0 : (BS == 32) ? h : (2 * h + q);                        \
-      const uint32_t mb_ = (stage_ptr_) + m_rd + blk_ * 256;                                 \
-      (dc_##_sc)[t][q] = lds_read_u16(mb_ + i * 2, t * 128);                                 \
-      (dc_##_zp)[t][q] = HAS_ZP ? lds_read_u8(mb_ + i, t * 128 + 64) : 8u;                   \
+    if (!ROW) {                                                                              \
+      _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                    \
+        const int blk_ = (BS == 64) ? 0 : (BS == 32) ? h : (2 * h + q);                      \
+        const uint32_t mb_ = (stage_ptr_) + m_rd + blk_ * 256;                               \
+        (dc_##_sc)[t][q] = lds_read_u16(mb_ + i * 2, t * 128);                               \
+        (dc_##_zp)[t][q] = HAS_ZP ? lds_read_u8(mb_ + i, t * 128 + 64) : 8u;                 \
+      }                                                                                      \
     }                                                                                        \
   }
-#define BLKQ4_MAKE_CONSTS(dc_)                            \
-  _Pragma("unroll") for (int t = 0; t < NT; ++t)          \
-  _Pragma("unroll") for (int q = 0; q < kMeta; ++q)(dc_)[t][q] = make_dequant_consts((dc_##_sc)[t][q], (dc_##_zp)[t][q])
+#define BLKQ4_MAKE_CONSTS(dc_)                                                                      \
+  if (!ROW) {                                                                                       \
+    _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                                \
+      _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                           \
+        (dc_)[t][q] = make_dequant_consts((dc_##_sc)[t][q], (dc_##_zp)[t][q]);                      \
+      }                                                                                             \
+    }                                                                                               \
+  }
+  // blocks along N: scales (2 x 16 bytes) and zero-points (16 bytes) of 16-row group 2h + jj_ of every
+  // fragment's column group, as they lie in memory
+#define BLKQ4_READ_ROW_META(jj_, stage_off_)                                                     \
+  if (ROW) {                                                                                     \
+    _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                             \
+      mrow_s[jj_][t][0] = lds_read_16((stage_off_) + msc_rd[t], (jj_) * 32);                     \
+      mrow_s[jj_][t][1] = lds_read_16((stage_off_) + msc_rd[t], (jj_) * 32 + 16);                \
+      if (HAS_ZP) mrow_z[jj_][t] = lds_read_16((stage_off_) + mzp_rd[t], (jj_) * 16);            \
+    }                                                                                            \
+  }
   // Piece y (0 .. 4*NT-1) of the conversion of word `w_` of every fragment into fragment buffer `dst_` is fp16
   // pair y % 4 of fragment y / 4.  Its three instructions depend on each other (and a packed instruction
   // that reads the result of the one before it costs a wait state), so two pieces are converted together,
@@ -281,13 +346,21 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   pt[y_] = as_half2((((((y_) % 4) >= 2) ? ((words_)[(y_) / 4][w_] >> 8) : (words_)[(y_) / 4][w_]) &      \
                      ((((y_) & 1) == 0) ? masks.lo_mask : masks.hi_mask)) |                               \
                     ((((y_) & 1) == 0) ? masks.magic_1024 : masks.magic_64))
-#define BLKQ4_PIECE_PA(dc_, q_, y_) \
-  pt[y_] = pt[y_] + ((((y_) & 1) == 0) ? (dc_)[(y_) / 4][q_].neg_c0 : (dc_)[(y_) / 4][q_].neg_c1)
-#define BLKQ4_PIECE_PM(dst_, dc_, q_, y_) wp[dst_][(y_) / 4][(y_) % 4] = pt[y_] * (dc_)[(y_) / 4][q_].scale2
+  // Blocks along N: word w_ of a lane's unit is rows 8 hh .. 8 hh + 7 (hh = w_ & 1) of 16-row group w_ / 2 of
+  // the lane's 32 rows; pair p has its zero-points in byte pair hh of zero-point word p and its scales in
+  // word 2 p + hh of the group (see blkq4_device.h for the packed order).
+#define BLKQ4_PIECE_PA(dc_, q_, w_, y_)                                                                       \
+  pt[y_] = pt[y_] + (ROW ? row_neg_c<HAS_ZP>(vec_word(mrow_z[(w_) >> 1][(y_) / 4], (y_) % 4), (y_) % 4, (w_)&1, rmasks) \
+                     : ((((y_) & 1) == 0) ? (dc_)[(y_) / 4][q_].neg_c0 : (dc_)[(y_) / 4][q_].neg_c1))
+#define BLKQ4_PIECE_PM(dst_, dc_, q_, w_, y_)                                                                \
+  wp[dst_][(y_) / 4][(y_) % 4] =                                                                             \
+      pt[y_] * (ROW ? as_half2(vec_word(mrow_s[(w_) >> 1][(y_) / 4][(2 * ((y_) % 4) + ((w_)&1)) >> 2],       \
+                                        (2 * ((y_) % 4) + ((w_)&1)) & 3))                                    \
+                    : (dc_)[(y_) / 4][q_].scale2)
 #define BLKQ4_PIECE(dst_, words_, w_, dc_, q_, y_) \
   BLKQ4_PIECE_AO(words_, w_, y_);                  \
-  BLKQ4_PIECE_PA(dc_, q_, y_);                     \
-  BLKQ4_PIECE_PM(dst_, dc_, q_, y_)
+  BLKQ4_PIECE_PA(dc_, q_, w_, y_);                 \
+  BLKQ4_PIECE_PM(dst_, dc_, q_, w_, y_)
 #define BLKQ4_WFRAG(slot_, t_) \
   __builtin_bit_cast(half8_t, half2x4_t{wp[slot_][t_][0], wp[slot_][t_][1], wp[slot_][t_][2], wp[slot_][t_][3]})
 
@@ -301,10 +374,12 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   uint32_t words[NT][4], nwords[NT][4];
   uint32_t dc_sc[NT][kMeta], dc_zp[NT][kMeta], ndc_sc[NT][kMeta], ndc_zp[NT][kMeta];
   DequantConsts dc[NT][kMeta], ndc[NT][kMeta];
+  uint4 mrow_s[2][NT][2], mrow_z[2][NT];  // blocks along N: meta of 16-row groups 2h (steps 0, 1) and 2h + 1 (steps 2, 3)
 
   {
     const uint32_t s0 = 0;
     BLKQ4_READ_B(words, dc, s0);
+    BLKQ4_READ_ROW_META(0, s0);
     BLKQ4_MAKE_CONSTS(dc);
 #pragma unroll
     for (int r = 0; r < RT; ++r) BLKQ4_READ_A1(af[0], s0, 0, r);
@@ -333,11 +408,11 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
             BLKQ4_PIECE_AO(nwords_, nw_, 2 * g2);                                                  \
             BLKQ4_PIECE_AO(nwords_, nw_, 2 * g2 + 1);                                              \
           }                                                                                        \
-          if (stage_slot(g2, 1, 2 * NT, kMfmas) == x_) BLKQ4_PIECE_PA(ndc_, nq_, 2 * g2);          \
-          if (stage_slot(g2, 2, 2 * NT, kMfmas) == x_) BLKQ4_PIECE_PA(ndc_, nq_, 2 * g2 + 1);      \
+          if (stage_slot(g2, 1, 2 * NT, kMfmas) == x_) BLKQ4_PIECE_PA(ndc_, nq_, nw_, 2 * g2);     \
+          if (stage_slot(g2, 2, 2 * NT, kMfmas) == x_) BLKQ4_PIECE_PA(ndc_, nq_, nw_, 2 * g2 + 1); \
           if (stage_slot(g2, 3, 2 * NT, kMfmas) == x_) {                                           \
-            BLKQ4_PIECE_PM(1 - (cur_), ndc_, nq_, 2 * g2);                                         \
-            BLKQ4_PIECE_PM(1 - (cur_), ndc_, nq_, 2 * g2 + 1);                                     \
+            BLKQ4_PIECE_PM(1 - (cur_), ndc_, nq_, nw_, 2 * g2);                                    \
+            BLKQ4_PIECE_PM(1 - (cur_), ndc_, nq_, nw_, 2 * g2 + 1);                                \
           }                                                                                        \
         }                                                                                          \
         _Pragma("unroll") for (int y = (lo_); y < (hi_); ++y) {                                    \
@@ -365,6 +440,7 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
     BLKQ4_PIN();
 
     // step 0: uses buffers 0; prepares step 1
+    BLKQ4_READ_ROW_META(1, sa);
     BLKQ4_STEP(0, sa, 1, words, 1, dc, 0, (kCopySteps == 4 ? kCut2 : 0), (kCopySteps == 4 ? kCut3 : 0), late_tile, late_stage);
     // step 1: uses buffers 1; prepares step 2
     BLKQ4_STEP(1, sa, 2, words, 2, dc, kMeta - 1, (kCopySteps == 4 ? kCut3 : 0), (kCopySteps == 4 ? kOps : 0), late_tile, late_stage);
@@ -373,6 +449,7 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
     block_barrier();
     // step 2: uses buffers 0; prepares step 3, reads the next tile's weights, starts the copies
     BLKQ4_READ_B(nwords, ndc, sn);
+    BLKQ4_READ_ROW_META(0, sn);
     BLKQ4_PIN();
     BLKQ4_STEP(0, sa, 3, words, 3, dc, kMeta - 1, 0, kCut1, copy_tile, copy_stage);
     // step 3: uses buffers 1; prepares step 0 of tile kt+1, finishes the copies
@@ -392,6 +469,7 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
 #undef BLKQ4_READ_A1
 #undef BLKQ4_READ_B
 #undef BLKQ4_MAKE_CONSTS
+#undef BLKQ4_READ_ROW_META
 #undef BLKQ4_PIECE
 #undef BLKQ4_PIECE_AO
 #undef BLKQ4_PIECE_PA
@@ -441,14 +519,14 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   }
 }
 
-template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW>
+template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW = false>
 int launch_one(const blkq4_gemm_args* a) {
   constexpr int BM = 32 * RT * WM;
   constexpr int kBN = 32 * NT * WN;
   const int m_tiles = (a->m + BM - 1) / BM;
   const int n_tiles = (a->n + kBN - 1) / kBN;
   const dim3 grid(static_cast<unsigned>(m_tiles) * n_tiles);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW>), grid, dim3(64 * (WM * WN + PW)), 0,
+  hipLaunchKernelGGL((gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW, ROW>), grid, dim3(64 * (WM * WN + PW)), 0,
                      static_cast<hipStream_t>(a->stream), static_cast<const uint8_t*>(a->a),
                      static_cast<const uint8_t*>(a->packed_w), static_cast<const uint8_t*>(a->scales),
                      static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c), a->m, a->n,
@@ -458,12 +536,6 @@ int launch_one(const blkq4_gemm_args* a) {
 
 template <int BS, bool HAS_ZP>
 int launch_rt(const blkq4_gemm_args* a) {
-  // rows per workgroup: no more than the problem has
-  if (a->m <= 32) return launch_one<BS, HAS_ZP, 1, 1, 1, 8, 0>(a);
-  if (a->m <= 64) return launch_one<BS, HAS_ZP, 2, 1, 1, 8, 0>(a);
-#ifdef BLKQ4_GEMM_SHAPE
-  return launch_one<BS, HAS_ZP, BLKQ4_GEMM_SHAPE>(a);
-#else
   // Problems with at least one 256 x 256 tile per compute unit: four waves of 256 x 64 each, the
   // fewest conversion instructions per MFMA (every register of a SIMD belongs to one wave, which
   // leaves no room for producer waves).  Smaller ones: 128 x 256 tiles, four waves of 128 x 64 plus
@@ -471,8 +543,20 @@ int launch_rt(const blkq4_gemm_args* a) {
   // (four waves of 128 x 32): twice the workgroups, each done in 0.6 of the time.
   constexpr int kComputeUnits = 256;
   const long tiles = static_cast<long>((a->m + 255) / 256) * ((a->n + 255) / 256);
-  if (tiles >= kComputeUnits) return launch_one<BS, HAS_ZP, 8, 2, 1, 4, 0>(a);
   const long small_tiles = static_cast<long>((a->m + 127) / 128) * ((a->n + 127) / 128);
+  if (!a->column_wise) {
+    // blocks along N (the streaming kernel takes the small row counts)
+    if (tiles >= kComputeUnits) return launch_one<BS, HAS_ZP, 8, 2, 1, 4, 0, true>(a);
+    if (small_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 4, 1, 1, 4, 4, true>(a);
+    return launch_one<BS, HAS_ZP, 4, 2, 1, 4, 4, true>(a);
+  }
+  // rows per workgroup: no more than the problem has
+  if (a->m <= 32) return launch_one<BS, HAS_ZP, 1, 1, 1, 8, 0>(a);
+  if (a->m <= 64) return launch_one<BS, HAS_ZP, 2, 1, 1, 8, 0>(a);
+#ifdef BLKQ4_GEMM_SHAPE
+  return launch_one<BS, HAS_ZP, BLKQ4_GEMM_SHAPE>(a);
+#else
+  if (tiles >= kComputeUnits) return launch_one<BS, HAS_ZP, 8, 2, 1, 4, 0>(a);
   if (small_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 4, 1, 1, 4, 4>(a);
   return launch_one<BS, HAS_ZP, 4, 2, 1, 4, 4>(a);
 #endif
@@ -487,6 +571,10 @@ int launch_bs(const blkq4_gemm_args* a) {
 
 extern "C" int blkq4_dev_gemm(const blkq4_gemm_args* a) {
   if (a->m < 1 || (a->n % 32) != 0 || a->n < 32 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
+  if (!a->column_wise && ((a->n % a->block_size) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 3u) != 0 ||
+                          (reinterpret_cast<uintptr_t>(a->zero_points) & 3u) != 0)) {
+    return static_cast<int>(hipErrorInvalidValue);  // the meta data are copied four bytes at a time
+  }
   // the async copies address A and W with 32-bit byte offsets from a per-tile base
   if (static_cast<uint64_t>(a->m) * a->k * 2 >= (1ull << 32) || static_cast<uint64_t>(a->k) * a->n / 2 >= (1ull << 32)) {
     return static_cast<int>(hipErrorInvalidValue);
