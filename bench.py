@@ -55,17 +55,20 @@ DESCRIPTION = {
 # HBM-side traffic per launch, measured with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (two runs of
 # this script, KiB per dispatch, mean over the dispatches of the kernel) and scaled by what the same counter
 # reads for the runtime's device-to-device copy of a 128 MiB buffer in the same run (FETCH_SIZE reads
-# 65 557 KiB for 131 072 KiB fetched: factor 2.0; WRITE_SIZE reads 131 072 KiB: factor 1.0).  The counters
+# 65 552 KiB for 131 072 KiB fetched: factor 2.0; WRITE_SIZE reads 131 072 KiB: factor 1.0).  The counters
 # sit between L2 and the memory fabric, so reads served by the Infinity Cache are included.  A script cannot
 # read these counters for itself; the figures are refreshed when a kernel changes.
-COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65557.0, "WRITE_SIZE": 1.0}
+COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65552.0, "WRITE_SIZE": 1.0}
 COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
-    "C4": (44090.3, 16384.0),
-    "C2": (5191.1, 8.0),
-    "C3": (16652.1, 344.0),
-    "C5": (860293.0, 229422.0),
-    "C5_prepack": (229442.0, 158496.0),
-    "C4r": (51758.9, 30282.2),
+    "C4": (44090.8, 16384.0),
+    "C2": (4413.0, 8.0),
+    "C3": (13867.8, 344.0),
+    "C5": (860310.0, 229376.0),
+    "C5_prepack": (229442.0, 158472.6),
+    "C4r": (44090.6, 16384.0),
+    "C2r": (4408.9, 8.0),
+    "C1": (856.7, 128.0),
+    "M128": (8649.5, 1024.0),
 }
 
 
