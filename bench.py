@@ -242,7 +242,9 @@ def bench_context(torch, capi, device, head_problem, steps, warmup):
     * the vendor library's plain fp16 GEMM (torch.matmul on an fp16 copy of the dequantized-size weight
       matrix, no 4-bit weights involved) on the headline shape;
     * the headline GEMM on all-zero activations and weights: same instruction stream, idle data paths --
-      the difference to the real run is what the clock loses under load."""
+      the difference to the real run is what the clock loses under load;
+    * a kernel that does nothing but back-to-back fp16 MFMAs (one wave per SIMD, all 256 compute units) on
+      random and on all-zero operands: the rate the chip sustains, which is the ceiling of any fp16 GEMM."""
     import ctypes
     from gemmlib_amd import build as _build
     out = {}
@@ -251,12 +253,20 @@ def bench_context(torch, capi, device, head_problem, steps, warmup):
     probe.blkq4_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                          ctypes.c_void_p, ctypes.c_void_p]
     scratch = torch.zeros(1 << 16, dtype=torch.int32, device=device)
+    probe.blkq4_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
 
     def stream_ptr():
         return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
     wall, evt, _ = timed_region(torch, [lambda: probe.blkq4_probe_empty(scratch.data_ptr(), stream_ptr())], steps, warmup)
     out["empty_kernel_us"] = round(evt / steps * 1e6, 3)
+    mfma_iters = 4000  # about 2 ms of MFMAs per launch, long enough for the clock to settle
+    for random_operands, key in ((1, "mfma_only_random_operands_tflops"), (0, "mfma_only_zero_operands_tflops")):
+        n_launch = 20
+        wall, evt, _ = timed_region(
+            torch, [lambda: probe.blkq4_probe_mfma(random_operands, mfma_iters, scratch.data_ptr(), stream_ptr())],
+            n_launch, 3)
+        out[key] = round(256 * 4 * mfma_iters * 8 * 32768.0 / (evt / n_launch) / 1e12, 1)
     m, k, n, bs, has_offsets, _ = CONFIGS["C2"]
     per_set = k * n // 2 + 2 * k * n // bs
     copies = INFINITY_CACHE_BYTES // per_set + 2

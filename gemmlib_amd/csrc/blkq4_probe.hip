@@ -1,7 +1,8 @@
 // Measurement aids for bench.py (their own small library, not part of the product's ABI): an empty
-// kernel, and a kernel that issues the weight-streaming kernel's memory requests and nothing else.  They
-// give the two floors that the GEMV figures are read against: what a graph node costs when it does
-// nothing, and what reading the packed weights and scales costs with this access pattern.
+// kernel, a kernel that issues the weight-streaming kernel's memory requests and nothing else, and a kernel
+// that does nothing but fp16 MFMAs.  They give what the figures are read against: what a graph node costs
+// when it does nothing, what reading the packed weights and scales costs with this access pattern, and the
+// MFMA rate the chip sustains on real operands (the clock it holds depends on the operands' bits).
 
 #include <hip/hip_runtime.h>
 
@@ -38,6 +39,45 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const uint4* __restr
   if (a == 0x12345678u) out[blockIdx.x] = a;  // keeps the loads alive, (almost) never stores
 }
 
+typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
+typedef float probe_float16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ unsigned mix_bits(unsigned x) {
+  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+  return x;
+}
+
+// One wave per SIMD, eight independent accumulators, back-to-back v_mfma_f32_32x32x16_f16 and nothing else.
+// RANDOM: operands are fp16 values of either sign in [0.125, 0.5) with random mantissas; otherwise zeros.
+template <bool RANDOM>
+__global__ __launch_bounds__(256) void mfma_kernel(float* out, int iters) {
+  probe_half8 a[8], b[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const unsigned r = mix_bits(threadIdx.x * 64 + s * 8 + e + blockIdx.x * 7919u);
+      a[s][e] = __builtin_bit_cast(_Float16, static_cast<unsigned short>(RANDOM ? (0x3000u | (r & 0x8fffu)) : 0u));
+      b[s][e] = __builtin_bit_cast(_Float16, static_cast<unsigned short>(RANDOM ? (0x3000u | ((r >> 16) & 0x8fffu)) : 0u));
+    }
+  }
+  probe_float16 acc[8];
+#pragma unroll
+  for (int n = 0; n < 8; ++n)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[n][e] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int n = 0; n < 8; ++n) acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[n], b[(3 * n + 1) & 7], acc[n], 0, 0, 0);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int n = 0; n < 8; ++n)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) sum += acc[n][e];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = sum;
+}
+
 }  // namespace
 
 #define PROBE_EXPORT extern "C" __attribute__((visibility("default")))
@@ -61,6 +101,19 @@ PROBE_EXPORT int blkq4_probe_stream(const void* packed_w, const void* scales, in
     hipLaunchKernelGGL((stream_kernel<8, false>), grid, block, 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint4*>(packed_w), static_cast<const uint16_t*>(nullptr),
                        static_cast<unsigned*>(scratch), n, k);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+// 256 workgroups of four waves, `iters` x 8 MFMAs per wave: 256 * 4 * iters * 8 * 32768 flop.
+// scratch: at least 256 * 256 * 4 bytes
+PROBE_EXPORT int blkq4_probe_mfma(int random_operands, int iters, void* scratch, void* stream) {
+  if (random_operands) {
+    hipLaunchKernelGGL(mfma_kernel<true>, dim3(256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<float*>(scratch), iters);
+  } else {
+    hipLaunchKernelGGL(mfma_kernel<false>, dim3(256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<float*>(scratch), iters);
   }
   return static_cast<int>(hipGetLastError());
 }
