@@ -18,16 +18,6 @@ __device__ __forceinline__ void async_copy_16(uint32_t lds_base, const void* bas
 __device__ __forceinline__ void async_copy_4_flat(uint32_t lds_base, const void* gptr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
 }
-// the same with lanes 0..31 only (the other lanes must be active when this is called)
-__device__ __forceinline__ void async_copy_4_flat_lo32(uint32_t lds_base, const void* gptr) {
-  uint64_t saved;
-  asm volatile(
-      "s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
-      "global_load_lds_dword %2, off\n\ts_mov_b64 exec, %0"
-      : "=&s"(saved)
-      : "s"(lds_base), "v"(gptr)
-      : "memory");
-}
 // LDS reads at byte address `addr` + `imm`.  `imm` is a compile-time constant applied as a pointer offset,
 // which the compiler folds into the instruction's offset field (it will not do that for an integer addition,
 // which may wrap); `addr` costs whatever the caller spends on it and nothing more.
@@ -53,7 +43,6 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
-__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 // s_barrier that the compiler may not move LDS accesses across, in either direction
 __device__ __forceinline__ void block_barrier() {
   asm volatile("" ::: "memory");
