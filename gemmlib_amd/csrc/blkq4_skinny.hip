@@ -6,7 +6,9 @@
 // deeply as possible and nothing serialises behind it:
 //   - a workgroup of 4, 8 or 16 waves owns 16 * NT output columns, 16 * MT rows and the whole K range; the
 //     waves split K in 128-deep slices, so every wave load is one 16-byte unit per lane: 16 columns x 4
-//     consecutive k-units = four contiguous 256-byte runs of the packed layout;
+//     consecutive k-units = four contiguous 256-byte runs of the packed layout.  With enough column tiles for
+//     every wave the chip holds (and few rows), the waves do not split K: each has column tiles of its own,
+//     streams all of K, and stores its sums itself: no barrier after the rows have arrived;
 //   - a wave keeps the weight units, scales and zero-points of DEPTH slices in flight and refills a
 //     slot as soon as it has consumed it (out-of-range slices wrap around to valid units and are
 //     multiplied by a zero scale, so the loop has no divergent loads);
@@ -21,7 +23,10 @@
 //   - the waves' partial tiles are summed through LDS (the space of the activation rows, once every wave
 //     is done with them) by all threads: no atomics, no scratch buffer;
 //   - more than 32 rows: the grid has one workgroup per (row group of 32, column group); the row groups
-//     of a column group run on the same XCD, so the weights they share are fetched into its L2 once.
+//     of a column group run on the same XCD, so the weights they share are fetched into its L2 once;
+//   - many more column groups than the chip holds workgroups: the grid is as large as the chip holds and a
+//     workgroup walks over several column groups, requesting the first slices of the next one while it
+//     finishes the current one.
 // Dequantization happens in registers (blkq4_dequant.h), for blocks along K (a scale per column and block
 // row) and along N (a scale per k, shared by BS columns, in the reference's packed order); accumulation
 // is fp32.
@@ -52,22 +57,28 @@ struct Slot {
   // the meta data (two 16-row groups of 32 + 16 bytes)
   uint4 rs[ROW ? NT : 1][4];
   uint4 rz[ROW ? NT : 1][2];
+
 };
 
-// kWaves: waves of the workgroup, which split K.  DEPTH: k slices (128 deep) a wave keeps in flight.  NT: 16-column tiles per wave that share one
-// activation operand.  MT: 16-row tiles of activations (M <= 16 * MT) that share one conversion of the
-// weights.  AM: where the activation rows are (see above).  kRowsWholeInLds: rows_log2 = log2 of the number
-// of rows kept in LDS, a power of two >= M, and the dynamic LDS size is red_bytes + (K * 2 << rows_log2).
-// kRowsPerSlotInLds: red_bytes + kWaves * DEPTH * 16 * MT * 256.
+// kWaves: waves of the workgroup.  kSplit: how many of them split K: all (kSplit = kWaves; their partial tiles
+// are summed through LDS) or none (kSplit = 1: every wave has NT column tiles of its own and all of K).
+// DEPTH: k slices (128 deep) a wave keeps in flight.  NT: 16-column tiles per wave that share one activation
+// operand.  MT: 16-row tiles of activations (M <= 16 * MT) that share one conversion of the weights.
+// AM: where the activation rows are (see above).  kRowsWholeInLds: rows_log2 = log2 of the number of rows kept
+// in LDS, a power of two >= M; kRowsPerSlotInLds: kWaves * DEPTH * 16 * MT * 256 bytes of slots.
+// kRefill: false for one column group (NT * kWaves / kSplit tiles) per workgroup; true for workgroups that walk
+// over the column groups cg, cg + cg_stride, ... (the partial tiles then live at red_offset, behind the rows,
+// which stay) and for waves that do not split K.
 // ROW: quantization blocks run along N (one k, BS columns); S and Z are then in the packed order
 // described in blkq4_device.h and the lane's column group decides which 64 + 32 bytes it fetches per unit.
-template <int BS, bool HAS_ZP, int DEPTH, int NT, int MT, int kWaves, int AM, bool ROW>
+template <int BS, bool HAS_ZP, int DEPTH, int NT, int MT, int kWaves, int AM, bool ROW, bool kRefill, int kSplit>
 __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t* __restrict__ A,
                                                                const uint4* __restrict__ W,
                                                                const uint16_t* __restrict__ S,
                                                                const uint8_t* __restrict__ Z,
                                                                uint16_t* __restrict__ C, int M_total, int N,
-                                                               int K, int rows_log2, int row_groups) {
+                                                               int K, int rows_log2, int row_groups,
+                                                               int cg_stride, uint32_t red_offset) {
   constexpr int kMeta = Slot<BS, NT, MT, AM, ROW>::kMeta;
   constexpr bool A_LDS = AM == kRowsWholeInLds;
   // weight / scale / zero-point requests of a slot
@@ -76,7 +87,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   constexpr int kSlotBytes = kSlotRows * 256;
   // the partial tiles of the final reduction reuse the LDS of the activation rows
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  float* red = reinterpret_cast<float*>(smem);
+  float* red = reinterpret_cast<float*>(smem + red_offset);
   const uint8_t* a_lds = smem;
 
   // Workgroup -> (row group of 16 * MT rows, group of NT column tiles).  Consecutive workgroups go to
@@ -84,11 +95,13 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   // group (they share its weights), then the next of four neighbouring column groups (they share the 128-byte
   // lines of the scale and zero-point rows, and their weights are contiguous), so that what is shared is
   // fetched into that XCD's L2 once.
-  const int col_groups = ((N >> 4) + NT - 1) / NT;
+  static_assert(kSplit == kWaves || kSplit == 1, "the waves split K among all of them or not at all");
+  constexpr int kTileWaves = kWaves / kSplit;  // waves (or sets of waves) with column tiles of their own
+  const int col_groups = ((N >> 4) + NT * kTileWaves - 1) / (NT * kTileWaves);
   const int wg = blockIdx.x;
   const int q = wg >> 3;
   const int rg = q % row_groups;
-  const int cg = 4 * ((wg & 7) + 8 * ((q / row_groups) >> 2)) + ((q / row_groups) & 3);
+  int cg = 4 * ((wg & 7) + 8 * ((q / row_groups) >> 2)) + ((q / row_groups) & 3);
   if (cg >= col_groups) return;  // the grid is rounded up to whole groups of 32 column groups
   const int m0 = rg * (16 * MT);
   const int M = min(16 * MT, M_total - m0);
@@ -101,18 +114,12 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   const int nl = lane & 15;  // column inside the tile (weights operand) / activation row (other operand)
   const int g = lane >> 4;   // which of the 4 k-units of a slice
   const int tiles = N >> 4;
-  // column this lane loads for tile t; a tile past the end (last workgroup only, when NT does not
-  // divide the tile count) re-reads the workgroup's first tile and is not stored
-  int n[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int tile = cg * NT + t;
-    n[t] = ((tile < tiles) ? tile : cg * NT) * 16 + nl;
-  }
   const DequantMasks masks = DequantMasks::make();
   const int units = K >> 5;             // 32-deep units
   const int slices = (units + 3) >> 2;  // 128-deep slices (the last one may be half full)
-  const int my_slices = (slices - wave + kWaves - 1) / kWaves;  // slices wave, wave + kWaves, ...
+  const int ws = (kSplit == 1) ? 0 : wave;  // this wave's slices are ws, ws + kSplit, ...
+  const int wt = (kSplit == 1) ? wave : 0;  // and its column tiles the wt-th NT of the column group
+  const int my_slices = (slices - ws + kSplit - 1) / kSplit;
 
   const int wrap_mask = (1 << (31 - __builtin_clz(units))) - 1;  // any index & wrap_mask is < units
 
@@ -148,17 +155,23 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     a_rd = row * 64;
     a_swz = (row >> 2) & 3;
   }
-  // a slice past the end wraps around to valid units (so every slot always issues the same loads)
-  // and gets a zero scale, which makes it contribute exactly 0
-#define BLKQ4_LOAD_SLOT(dst_, d_, slice_)                                                        \
+  // a slice past the end wraps around to valid units (so every slot always issues the same loads); its
+  // scales are zeroed when the slot is consumed (not here: that would wait for the load right after
+  // requesting it), which makes it contribute exactly 0
+#define BLKQ4_LOAD_SLOT(dst_, d_, cg_, slice_, keep_)                                                \
   {                                                                                            \
+    /* column this lane loads for tile t of column group cg_; a tile past the end (last column  */ \
+    /* group only, when NT does not divide the tile count) re-reads the group's first tile and  */ \
+    /* is not stored                                                                            */ \
+    int n[NT];                                                                                 \
+    _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                           \
+      const int tile_ = ((cg_) * kTileWaves + wt) * NT + t;                                    \
+      n[t] = (((tile_ < tiles) ? tile_ : (cg_) * (kTileWaves * NT)) * 16 + nl) & (keep_);      \
+    }                                                                                          \
     const int ks_ = 4 * (slice_) + g;                                                          \
     const bool ok_ = ks_ < units;                                                              \
-    const int ksg_ = ok_ ? ks_ : (ks_ & wrap_mask);                                            \
+    const int ksg_ = (ok_ ? ks_ : (ks_ & wrap_mask)) & (keep_);                                \
     const int b_ = (BS == 64) ? (ksg_ >> 1) : (BS == 32) ? ksg_ : (2 * ksg_);                  \
-    /* the scales of a slice past the end are zeroed with a mask, not a select: a select lets the   */ \
-    /* compiler skip the load, and the waits below count every load of a slot                       */ \
-    const uint32_t okm_ = ok_ ? 0xffffffffu : 0u;                                              \
     if (AM == kRowsPerSlotInLds) {                                                             \
       /* copy q: LDS bytes [1024 q, 1024 q + 1024) of the slot, lane l the 16 bytes at 16 l; */ \
       /* requested before the slot's weights, so whoever has the weights has the rows        */ \
@@ -168,7 +181,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
         const int ug_ = (u_ < units) ? u_ : (u_ & wrap_mask);                                  \
         const int row_ = rr_ % kSlotRows;                                                      \
         const int chunk_ = (lane & 3) ^ ((row_ >> 2) & 3);                                     \
-        async_copy_16(lds0 + (wave * DEPTH + (d_)) * kSlotBytes + q * 1024, A,                 \
+        async_copy_16(__builtin_amdgcn_readfirstlane(lds0 + (wave * DEPTH + (d_)) * kSlotBytes + q * 1024), A, \
                       (static_cast<uint32_t>(min(row_, M - 1)) * K + ug_ * 32 + chunk_ * 8) * 2); \
       }                                                                                        \
     }                                                                                          \
@@ -177,8 +190,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       if (ROW) {                                                                               \
         const size_t mi_ = static_cast<size_t>(n[t] / BS) * K + static_cast<size_t>(ksg_) * 32; \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                        \
-          const uint4 v_ = reinterpret_cast<const uint4*>(S + mi_)[q];                         \
-          (dst_).rs[ROW ? t : 0][q] = make_uint4(v_.x & okm_, v_.y & okm_, v_.z & okm_, v_.w & okm_); \
+          (dst_).rs[ROW ? t : 0][q] = reinterpret_cast<const uint4*>(S + mi_)[q];              \
         }                                                                                      \
         if (HAS_ZP) {                                                                          \
           _Pragma("unroll") for (int q = 0; q < 2; ++q) {                                      \
@@ -188,15 +200,16 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       } else {                                                                                 \
         _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                    \
           const size_t mi_ = static_cast<size_t>(b_ + q) * N + n[t];                         \
-          const uint32_t sc_ = S[mi_];                                                         \
-          (dst_).sc[t][ROW ? 0 : q] = sc_ & okm_;                                              \
+          (dst_).sc[t][ROW ? 0 : q] = S[mi_];                                                  \
           (dst_).zp[t][ROW ? 0 : q] = HAS_ZP ? static_cast<uint32_t>(Z[mi_]) : 8u;             \
         }                                                                                      \
       }                                                                                        \
     }                                                                                          \
   }
+  // A wave's local slices are li = 0 .. my_slices - 1 (slice ws + kSplit * li), taken DEPTH at a time; the
+  // slots past my_slices in the last round wrap around and are zeroed.
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d) BLKQ4_LOAD_SLOT(slot[d], d, wave + d * kWaves);
+  for (int d = 0; d < DEPTH; ++d) BLKQ4_LOAD_SLOT(slot[d], d, cg, ws + kSplit * d, -1);
   if (A_LDS) {
     // everything but the requests of the ring just issued has landed: this wave's share of the rows
     constexpr int kRing = DEPTH * kLoads;
@@ -204,13 +217,58 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     __syncthreads();
   }
 
-  for (int i0 = 0; i0 < my_slices; i0 += DEPTH) {
+  // Sums the waves' partial tiles of column group `cgx` through LDS and stores the result: every wave is
+  // done with the rows (when the partial tiles share their space) and with reading the partial tiles of
+  // the column group before.
+  auto flush = [&](int cgx) {
+    if (kSplit == 1) {
+      // a wave has whole sums: lane L holds columns 4 (L >> 4) .. + 3 of tile t, row 16 mt + (L & 15)
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      const int li = i0 + d;  // local slice index; slice = wave + 4*li
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const int tile = (cgx * kTileWaves + wt) * NT + t;
+          const int row = 16 * mt + nl;
+          if (row < M && tile < tiles) {
+            const uint32_t lo = float_to_half_bits(acc[t][mt][0]) | (static_cast<uint32_t>(float_to_half_bits(acc[t][mt][1])) << 16);
+            const uint32_t hi = float_to_half_bits(acc[t][mt][2]) | (static_cast<uint32_t>(float_to_half_bits(acc[t][mt][3])) << 16);
+            *reinterpret_cast<uint2*>(C + static_cast<size_t>(row) * N + tile * 16 + 4 * g) = make_uint2(lo, hi);
+          }
+          acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+      return;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) red[(((wave * NT + t) * MT + mt) * 64 + lane) * 4 + e] = acc[t][mt][e];
+        acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+      }
+    __syncthreads();
+    // value v = (tile t, row tile mt, lane L, element e) of the partial tiles: output row 16 mt + (L & 15),
+    // column 4 (L >> 4) + e of tile t; every thread sums a few of them over the waves
+    for (int v = tid; v < NT * MT * 256; v += 64 * kWaves) {
+      float r = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) r += red[w * (NT * MT * 256) + v];
+      const int t = v / (MT * 256), mt = (v >> 8) % MT, L = (v >> 2) & 63, e = v & 3;
+      const int row = 16 * mt + (L & 15);
+      if (row < M && cgx * NT + t < tiles) {
+        C[static_cast<size_t>(row) * N + cgx * (16 * NT) + 16 * t + 4 * (L >> 4) + e] = float_to_half_bits(r);
+      }
+    }
+  };
+
+  // converts slot d, which holds local slice li, and multiplies it with the rows
+  auto consume = [&](int d, int li) {
+    const Slot<BS, NT, MT, AM, ROW>& cur = slot[d];
+    const uint32_t okm = (4 * (ws + kSplit * li) + g < units) ? 0xffffffffu : 0u;
       half8_t af[MT][4];
       if (A_LDS) {
-        const int ks = 4 * (wave + kWaves * li) + g;
+        const int ks = 4 * (ws + kSplit * li) + g;
         const int ksg = (ks < units) ? ks : (ks & wrap_mask);
         const uint8_t* ap = a_lds + (static_cast<uint32_t>(ksg) << (6 + rows_log2)) + a_rd;
 #pragma unroll
@@ -220,10 +278,9 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
             af[mt][j] = as_half8(*reinterpret_cast<const uint4*>(ap + mt * 1024 + ((j ^ a_swz) * 16)));
           }
       } else {
-        // the rows of this slot were requested before its weights; younger than them are those weights and
-        // everything the other DEPTH - 1 slots have requested since
-        constexpr int kYounger = kLoads + (DEPTH - 1) * (4 * MT + kLoads);
-        wait_vmcnt<(kYounger < 63 ? kYounger : 63)>();
+        // the rows of this slot were requested before its weights
+        // (in-order completion: once one of the slot's weight words is here, so are the rows)
+        asm volatile("" ::: "memory");
         const uint8_t* ap = a_lds + a_rd + d * kSlotBytes;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -234,11 +291,11 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       }
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        const uint32_t words[4] = {slot[d].w[t].x, slot[d].w[t].y, slot[d].w[t].z, slot[d].w[t].w};
+        const uint32_t words[4] = {cur.w[t].x, cur.w[t].y, cur.w[t].z, cur.w[t].w};
         DequantConsts dc[kMeta];
         if (!ROW) {
 #pragma unroll
-          for (int q = 0; q < kMeta; ++q) dc[q] = make_dequant_consts(slot[d].sc[t][ROW ? 0 : q], slot[d].zp[t][ROW ? 0 : q]);
+          for (int q = 0; q < kMeta; ++q) dc[q] = make_dequant_consts(cur.sc[t][ROW ? 0 : q] & okm, cur.zp[t][ROW ? 0 : q]);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -249,15 +306,15 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
             // 32-bit word 2 i + hh of the group and its zero-points in byte pair hh of word i
             constexpr int kRowSlot = ROW ? 1 : 0;
             const int hh = j & 1;
-            const uint4 s0 = slot[d].rs[kRowSlot * t][2 * (j >> 1)], s1 = slot[d].rs[kRowSlot * t][2 * (j >> 1) + 1];
+            const uint4 s0 = cur.rs[kRowSlot * t][2 * (j >> 1)], s1 = cur.rs[kRowSlot * t][2 * (j >> 1) + 1];
             const uint32_t sw[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-            const uint4 zq = HAS_ZP ? slot[d].rz[kRowSlot * t][j >> 1] : make_uint4(0, 0, 0, 0);
+            const uint4 zq = HAS_ZP ? cur.rz[kRowSlot * t][j >> 1] : make_uint4(0, 0, 0, 0);
             const uint32_t zw[4] = {zq.x, zq.y, zq.z, zq.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const uint32_t zpair = HAS_ZP ? ((zw[i] >> (8 * hh)) & 0x00ff00ffu) : 0x00080008u;
               const uint32_t src = (i >= 2) ? y : words[j];
-              const half2_t s2 = as_half2(sw[2 * i + hh]);
+              const half2_t s2 = as_half2(sw[2 * i + hh] & okm);
               if ((i & 1) == 0) {
                 p[i] = (as_half2((src & masks.lo_mask) | masks.magic_1024) + as_half2(0xE400E400u | zpair)) * s2;
               } else {
@@ -280,32 +337,47 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
           }
         }
       }
-      if (i0 + DEPTH < my_slices) BLKQ4_LOAD_SLOT(slot[d], d, wave + kWaves * (li + DEPTH));
+  };
+
+  if (!kRefill) {
+    // one column group per workgroup: a slot is refilled only while the wave has slices left
+    for (int i0 = 0; i0 < my_slices; i0 += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        consume(d, i0 + d);
+        if (i0 + DEPTH < my_slices) BLKQ4_LOAD_SLOT(slot[d], d, cg, ws + kSplit * (i0 + d + DEPTH), -1);
+      }
     }
+    flush(cg);
+    return;
+  }
+  // A workgroup that walks over several column groups.  While a round is consumed, every slot is refilled
+  // with the same slot of the round after it: the next one of this column group, else the first one of the
+  // workgroup's next column group, else (nothing left) every lane asks for one and the same unit, unused.  So
+  // every round issues the same requests in the same order and the compiler's waits are exact; behind a
+  // conditional refill it waits for everything outstanding, the refills just issued included.
+  const int rounds = (my_slices + DEPTH - 1) / DEPTH;
+  while (cg < col_groups) {
+    const int next_cg = cg + cg_stride;
+    for (int r = 0; r < rounds; ++r) {
+      const int i0 = r * DEPTH;
+      const bool more = r + 1 < rounds;
+      const bool next_group = !more && next_cg < col_groups;
+      const int ld_cg = next_group ? next_cg : cg;
+      const int ld_i0 = more ? i0 + DEPTH : next_group ? 0 : i0;
+      const int keep = (more || next_group) ? -1 : 0;  // 0: every lane asks for the very first unit instead
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        consume(d, i0 + d);
+        BLKQ4_LOAD_SLOT(slot[d], d, ld_cg, ws + kSplit * (ld_i0 + d), keep);
+        // the refill is requested here, not together with the others at the end of the round
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    flush(cg);
+    cg = next_cg;
   }
 #undef BLKQ4_LOAD_SLOT
-
-  // cross-wave reduction through LDS (which holds activation rows until every wave is done with them)
-  __syncthreads();
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) red[(((wave * NT + t) * MT + mt) * 64 + lane) * 4 + e] = acc[t][mt][e];
-  __syncthreads();
-  // value v = (tile t, row tile mt, lane L, element e) of the partial tiles: output row 16 mt + (L & 15),
-  // column 4 (L >> 4) + e of tile t; every thread sums a few of them over the waves
-  for (int v = tid; v < NT * MT * 256; v += 64 * kWaves) {
-    float r = 0.f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) r += red[w * (NT * MT * 256) + v];
-    const int t = v / (MT * 256), mt = (v >> 8) % MT, L = (v >> 2) & 63, e = v & 3;
-    const int row = 16 * mt + (L & 15);
-    if (row < M && cg * NT + t < tiles) {
-      C[static_cast<size_t>(row) * N + cg * (16 * NT) + 16 * t + 4 * (L >> 4) + e] = float_to_half_bits(r);
-    }
-  }
 }
 
 // The kernel is bound by instruction issue as much as by the weight stream, so what matters is how
@@ -314,10 +386,13 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 // rows less often, which weighs more the more rows there are.
 constexpr size_t kMaxLdsBytes = 160 * 1024;
 constexpr int kStreamingMaxRows = 1024;
+constexpr int kComputeUnits = 256;
+constexpr int kIndependentMinTiles = 896;
+constexpr size_t kIndependentMaxRowBytes = 32 * 1024;
+constexpr int kPersistentFactor = 2;  // column groups per workgroup from which on workgroups walk
 
 
 void choose_shape(int m, int n, int* nt, int* depth) {
-  constexpr int kComputeUnits = 256;
   const int tiles = n / 16;
   const float a_weight = (m > 4) ? 0.2f : 0.05f;  // cost of fetching the activations relative to one tile's work
   float best = 0.f;
@@ -338,9 +413,9 @@ void choose_shape(int m, int n, int* nt, int* depth) {
 
 // One kernel instantiation: raises its dynamic-LDS limit once, then launches `row_groups` row groups of
 // 16 * MT rows each.
-template <int BS, bool HAS_ZP, bool ROW, int DEPTH, int NT, int MT, int kWaves, int AM>
+template <int BS, bool HAS_ZP, bool ROW, int DEPTH, int NT, int MT, int kWaves, int AM, int kSplit = kWaves>
 int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
-  constexpr size_t kRedBytes = static_cast<size_t>(kWaves) * NT * MT * 64 * 4 * 4;
+  constexpr size_t kRedBytes = (kSplit == 1) ? 0 : static_cast<size_t>(kWaves) * NT * MT * 64 * 4 * 4;
   constexpr size_t kPerSlotBytes = static_cast<size_t>(kWaves) * DEPTH * 16 * MT * 256;
   static_assert(kRedBytes <= kMaxLdsBytes, "partial tiles do not fit in LDS");
   static_assert(AM != kRowsPerSlotInLds || kPerSlotBytes <= kMaxLdsBytes, "slots do not fit in LDS");
@@ -348,18 +423,72 @@ int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
   const size_t a_bytes = AM == kRowsWholeInLds ? ((((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023})
                          : AM == kRowsPerSlotInLds ? kPerSlotBytes
                                                    : 0;
-  const size_t lds_bytes = a_bytes > kRedBytes ? a_bytes : kRedBytes;
-  auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW>;
-  static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
-  if (attr != hipSuccess) return static_cast<int>(attr);
-  const int col_groups = (a->n / 16 + NT - 1) / NT;
-  const unsigned grid = static_cast<unsigned>((col_groups + 31) / 32) * 32u * static_cast<unsigned>(row_groups);
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * kWaves), lds_bytes, static_cast<hipStream_t>(a->stream),
-                     static_cast<const uint16_t*>(a->a), static_cast<const uint4*>(a->packed_w),
-                     static_cast<const uint16_t*>(a->scales), static_cast<const uint8_t*>(a->zero_points),
-                     static_cast<uint16_t*>(a->c), a->m, a->n, a->k, rows_log2, row_groups);
-  return static_cast<int>(hipGetLastError());
+  constexpr int kGroupTiles = NT * (kWaves / kSplit);
+  const int col_groups = (a->n / 16 + kGroupTiles - 1) / kGroupTiles;
+  int cg_stride = (col_groups + 31) / 32 * 32;  // one column group per workgroup
+  size_t lds_bytes = a_bytes > kRedBytes ? a_bytes : kRedBytes;
+  size_t red_offset = 0;
+  // Many more workgroups than the chip holds at once: a workgroup then walks over several column groups
+  // (cg, cg + cg_stride, ...) and requests the first slices of the next one while it finishes the current
+  // one, so only the first column group of a workgroup waits for its weights with nothing else to do.
+  // The partial tiles then get LDS of their own: the rows stay where they are for the next column group.
+  // (not the sixteen-wave kernel for blocks along N: its walking variant does not fit in 128 registers)
+  constexpr bool kMayWalk = !(ROW && kWaves == 16);
+  if (kMayWalk && a_bytes + kRedBytes <= kMaxLdsBytes) {
+    const int by_lds = static_cast<int>(kMaxLdsBytes / (a_bytes + kRedBytes));
+    const int by_waves = 32 / kWaves;
+    const int resident = kComputeUnits * (by_lds < by_waves ? by_lds : by_waves);
+    int stride = (resident / row_groups) / 32 * 32;
+    if (stride < 32) stride = 32;
+    if (cg_stride >= kPersistentFactor * stride) {
+      cg_stride = stride;
+      lds_bytes = a_bytes + kRedBytes;
+      red_offset = a_bytes;
+    }
+  }
+  const unsigned grid = static_cast<unsigned>(cg_stride) * static_cast<unsigned>(row_groups);
+  // workgroups walk over several column groups, or waves stream all of K by themselves
+  const bool refill = cg_stride < col_groups || kSplit == 1;
+  auto launch = [&](auto* kernel, hipError_t attr) {
+    if (attr != hipSuccess) return static_cast<int>(attr);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * kWaves), lds_bytes, static_cast<hipStream_t>(a->stream),
+                       static_cast<const uint16_t*>(a->a), static_cast<const uint4*>(a->packed_w),
+                       static_cast<const uint16_t*>(a->scales), static_cast<const uint8_t*>(a->zero_points),
+                       static_cast<uint16_t*>(a->c), a->m, a->n, a->k, rows_log2, row_groups, cg_stride,
+                       static_cast<uint32_t>(red_offset));
+    return static_cast<int>(hipGetLastError());
+  };
+  if (refill) {
+    auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, true, kSplit>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
+    return launch(kernel, attr);
+  }
+  if constexpr (kSplit == 1) {
+    return static_cast<int>(hipErrorInvalidValue);  // not reached
+  } else {
+    auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, false, kSplit>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
+    return launch(kernel, attr);
+  }
+}
+
+// M <= 16, enough column tiles to give every wave the chip can hold one of its own, and rows small enough for
+// several workgroups per compute unit: the waves do not split K, each streams all of K for its own tile:
+// no sums across waves, no barriers, and a ring that stays full from the first slice to the last.
+template <int BS, bool HAS_ZP, bool ROW>
+bool launch_independent_waves(const blkq4_gemm_args* a, int* status) {
+  int rows_log2 = 0;
+  while ((1 << rows_log2) < a->m) ++rows_log2;
+  const size_t a_bytes = (((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023};
+  if (a->n / 16 < kIndependentMinTiles || a_bytes > kIndependentMaxRowBytes ||
+      (reinterpret_cast<uintptr_t>(a->c) & 7u) != 0) {
+    return false;
+  }
+  constexpr int kD = ROW ? 4 : 8;
+  *status = launch_kernel<BS, HAS_ZP, ROW, kD, 1, 1, 4, kRowsWholeInLds, 1>(a, rows_log2);
+  return true;
 }
 
 // M <= 16: one row tile; the waves of a workgroup split K.
@@ -395,13 +524,14 @@ int launch_shape(const blkq4_gemm_args* a) {
   if (a->m > 16) {
     // Every workgroup fetches the 32 rows of its group for all of K, so wide workgroups (more column tiles)
     // mean less activation traffic; but there should be a workgroup for every compute unit.
-    constexpr int kComputeUnits = 256;
-    const int row_groups = (a->m + 31) / 32;
+      const int row_groups = (a->m + 31) / 32;
     const long tiles = static_cast<long>(a->n / 16) * row_groups;
     if (tiles >= 4 * kComputeUnits) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 4>(a, row_groups);
     if (tiles >= 2 * kComputeUnits) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 2>(a, row_groups);
     return launch_rows<BS, HAS_ZP, ROW, 1>(a, row_groups);
   }
+  int status;
+  if (launch_independent_waves<BS, HAS_ZP, ROW>(a, &status)) return status;
   int nt, depth;
   choose_shape(a->m, a->n, &nt, &depth);
   if (ROW) {

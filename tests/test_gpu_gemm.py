@@ -80,7 +80,16 @@ LONG_K_CASES = [
 ]
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + LONG_K_CASES)
+# very wide N in the streaming kernel: few rows, where every wave streams all of K for a column tile of its own
+# (several rounds of its ring, K that ends inside a slice), and more rows, where a workgroup walks over
+# several column groups (rows whole in LDS, rows staged per slice, row groups of 32)
+VERY_WIDE_CASES = [
+    (64, False, 1, 14336, 4096), (32, True, 2, 16416, 4160), (16, True, 4, 28672, 320), (64, True, 1, 14336, 8320),
+    (64, True, 8, 32800, 4096), (32, True, 16, 16416, 8256), (32, True, 96, 5440, 4160), (16, False, 12, 28672, 1088),
+]
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + LONG_K_CASES + VERY_WIDE_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
 

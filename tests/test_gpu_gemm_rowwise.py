@@ -46,7 +46,14 @@ TILE_CASES = [
 ]
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EDGE_CASES + TILE_CASES)
+# very wide N in the streaming kernel: waves with a column tile of their own and all of K, and workgroups that
+# walk over several column groups
+VERY_WIDE_CASES = [
+    (64, False, 1, 14336, 4096), (32, True, 2, 16384, 2112), (16, True, 8, 28672, 1088), (64, True, 16, 16384, 8256),
+]
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EDGE_CASES + TILE_CASES + VERY_WIDE_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     rng = np.random.default_rng(m * 131 + n * 17 + k + bs + has_offsets)
     kat = oracle.kat_generate(bs, False, k, n, has_offsets)
