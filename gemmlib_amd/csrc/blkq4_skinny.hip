@@ -123,6 +123,25 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 
   const int wrap_mask = (1 << (31 - __builtin_clz(units))) - 1;  // any index & wrap_mask is < units
 
+  // Addresses are a wave-uniform 64-bit part (slice and column tile: scalar arithmetic) plus a 32-bit part
+  // of the lane that never changes: (k-unit of the slice g, column nl).  Only in the last slice, when it has
+  // rem < 4 units, the lanes past the end ask for unit g % rem instead (their scales are zeroed when the slot
+  // is consumed), and a slot past the wave's last slice asks for the last slice once more.
+  constexpr int kBlocksPerSlice = (BS == 64) ? 2 : (BS == 32) ? 4 : 8;
+  const int rem = units & 3;
+  const int last_slice = slices - 1;
+  const int g_alt = (rem == 0) ? g : (rem == 1) ? 0 : (rem == 2) ? (g & 1) : (g == 3 ? 0 : g);
+  uint32_t w_lane[2], m_lane[2], a_lane[2];  // [1]: in a last slice that is not full
+#pragma unroll
+  for (int v = 0; v < 2; ++v) {
+    const int gx = v ? g_alt : g;
+    w_lane[v] = static_cast<uint32_t>(gx * N + nl) * 16u;  // bytes into the packed weights
+    // elements into the scales and the zero-points
+    m_lane[v] = ROW ? static_cast<uint32_t>(gx * 32)
+                    : static_cast<uint32_t>(((BS == 64) ? (gx >> 1) : (BS == 32) ? gx : 2 * gx) * N + nl);
+  }
+  const uint32_t ok_last = (rem == 0 || g < rem) ? 0xffffffffu : 0u;
+
   float4_t acc[NT][MT];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
@@ -155,29 +174,24 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     a_rd = row * 64;
     a_swz = (row >> 2) & 3;
   }
-  // a slice past the end wraps around to valid units (so every slot always issues the same loads); its
-  // scales are zeroed when the slot is consumed (not here: that would wait for the load right after
-  // requesting it), which makes it contribute exactly 0
+  a_lane[0] = (static_cast<uint32_t>(g) << (6 + rows_log2)) + a_rd;
+  a_lane[1] = (static_cast<uint32_t>(g_alt) << (6 + rows_log2)) + a_rd;
+  // a slot past the end asks for valid units (so every slot always issues the same loads); its scales are
+  // zeroed when the slot is consumed (not here: that would wait for the load right after requesting it),
+  // which makes it contribute exactly 0
 #define BLKQ4_LOAD_SLOT(dst_, d_, cg_, slice_, keep_)                                                \
   {                                                                                            \
-    /* column this lane loads for tile t of column group cg_; a tile past the end (last column  */ \
-    /* group only, when NT does not divide the tile count) re-reads the group's first tile and  */ \
-    /* is not stored                                                                            */ \
-    int n[NT];                                                                                 \
-    _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                           \
-      const int tile_ = ((cg_) * kTileWaves + wt) * NT + t;                                    \
-      n[t] = (((tile_ < tiles) ? tile_ : (cg_) * (kTileWaves * NT)) * 16 + nl) & (keep_);      \
-    }                                                                                          \
-    const int ks_ = 4 * (slice_) + g;                                                          \
-    const bool ok_ = ks_ < units;                                                              \
-    const int ksg_ = (ok_ ? ks_ : (ks_ & wrap_mask)) & (keep_);                                \
-    const int b_ = (BS == 64) ? (ksg_ >> 1) : (BS == 32) ? ksg_ : (2 * ksg_);                  \
+    const int sl_ = min((slice_), last_slice);                                                 \
+    const bool alt_ = rem != 0 && sl_ == last_slice;                                           \
+    const uint32_t wl_ = alt_ ? w_lane[1] : w_lane[0];                                         \
+    const uint32_t ml_ = alt_ ? m_lane[1] : m_lane[0];                                         \
+    const size_t keep64_ = static_cast<size_t>(static_cast<long long>(keep_));                 \
     if (AM == kRowsPerSlotInLds) {                                                             \
       /* copy q: LDS bytes [1024 q, 1024 q + 1024) of the slot, lane l the 16 bytes at 16 l; */ \
       /* requested before the slot's weights, so whoever has the weights has the rows        */ \
       _Pragma("unroll") for (int q = 0; q < 4 * MT; ++q) {                                     \
         const int rr_ = 16 * q + (lane >> 2);            /* (unit, row) index inside the slot */ \
-        const int u_ = 4 * (slice_) + rr_ / kSlotRows;                                         \
+        const int u_ = 4 * sl_ + rr_ / kSlotRows;                                              \
         const int ug_ = (u_ < units) ? u_ : (u_ & wrap_mask);                                  \
         const int row_ = rr_ % kSlotRows;                                                      \
         const int chunk_ = (lane & 3) ^ ((row_ >> 2) & 3);                                     \
@@ -186,22 +200,32 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       }                                                                                        \
     }                                                                                          \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                           \
-      (dst_).w[t] = W[static_cast<size_t>(ksg_) * N + n[t]];                                  \
+      /* tile t of column group cg_; a tile past the end (last column group only, when the group's */ \
+      /* tile count does not divide the number of tiles) re-reads the group's first tile and is    */ \
+      /* not stored                                                                                */ \
+      const int tile_ = ((cg_) * kTileWaves + wt) * NT + t;                                    \
+      const int tu_ = (tile_ < tiles) ? tile_ : (cg_) * (kTileWaves * NT);                     \
+      const size_t wu_ = ((static_cast<size_t>(4 * sl_) * N + tu_ * 16) * 16) & keep64_;       \
+      (dst_).w[t] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(W) + wu_ + wl_); \
       if (ROW) {                                                                               \
-        const size_t mi_ = static_cast<size_t>(n[t] / BS) * K + static_cast<size_t>(ksg_) * 32; \
+        const size_t mu_ = (static_cast<size_t>(tu_ * 16 / BS) * K + sl_ * 128) & keep64_;     \
+        const char* sp_ = reinterpret_cast<const char*>(S) + mu_ * 2 + ml_ * 2;                \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                        \
-          (dst_).rs[ROW ? t : 0][q] = reinterpret_cast<const uint4*>(S + mi_)[q];              \
+          (dst_).rs[ROW ? t : 0][q] = reinterpret_cast<const uint4*>(sp_)[q];                  \
         }                                                                                      \
         if (HAS_ZP) {                                                                          \
+          const char* zp_ = reinterpret_cast<const char*>(Z) + mu_ + ml_;                      \
           _Pragma("unroll") for (int q = 0; q < 2; ++q) {                                      \
-            (dst_).rz[ROW ? t : 0][q] = reinterpret_cast<const uint4*>(Z + mi_)[q];            \
+            (dst_).rz[ROW ? t : 0][q] = reinterpret_cast<const uint4*>(zp_)[q];                \
           }                                                                                    \
         }                                                                                      \
       } else {                                                                                 \
         _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                    \
-          const size_t mi_ = static_cast<size_t>(b_ + q) * N + n[t];                         \
-          (dst_).sc[t][ROW ? 0 : q] = S[mi_];                                                  \
-          (dst_).zp[t][ROW ? 0 : q] = HAS_ZP ? static_cast<uint32_t>(Z[mi_]) : 8u;             \
+          const size_t mu_ = (static_cast<size_t>(kBlocksPerSlice * sl_ + q) * N + tu_ * 16) & keep64_; \
+          (dst_).sc[t][ROW ? 0 : q] =                                                          \
+              *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(S) + mu_ * 2 + ml_ * 2); \
+          (dst_).zp[t][ROW ? 0 : q] =                                                          \
+              HAS_ZP ? static_cast<uint32_t>(*(reinterpret_cast<const uint8_t*>(Z) + mu_ + ml_)) : 8u; \
         }                                                                                      \
       }                                                                                        \
     }                                                                                          \
@@ -265,12 +289,14 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   // converts slot d, which holds local slice li, and multiplies it with the rows
   auto consume = [&](int d, int li) {
     const Slot<BS, NT, MT, AM, ROW>& cur = slot[d];
-    const uint32_t okm = (4 * (ws + kSplit * li) + g < units) ? 0xffffffffu : 0u;
+    const int slice = ws + kSplit * li;
+    const int sl = min(slice, last_slice);
+    const bool alt = rem != 0 && sl == last_slice;
+    const uint32_t full = (slice < last_slice || (slice == last_slice && rem == 0)) ? 0xffffffffu : 0u;  // uniform
+    const uint32_t okm = full | ((slice == last_slice) ? ok_last : 0u);
       half8_t af[MT][4];
       if (A_LDS) {
-        const int ks = 4 * (ws + kSplit * li) + g;
-        const int ksg = (ks < units) ? ks : (ks & wrap_mask);
-        const uint8_t* ap = a_lds + (static_cast<uint32_t>(ksg) << (6 + rows_log2)) + a_rd;
+        const uint8_t* ap = a_lds + (static_cast<uint32_t>(4 * sl) << (6 + rows_log2)) + (alt ? a_lane[1] : a_lane[0]);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
