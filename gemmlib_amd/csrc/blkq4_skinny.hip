@@ -413,8 +413,6 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 constexpr size_t kMaxLdsBytes = 160 * 1024;
 constexpr int kStreamingMaxRows = 1024;
 constexpr int kComputeUnits = 256;
-constexpr int kIndependentMinTiles = 896;
-constexpr size_t kIndependentMaxRowBytes = 32 * 1024;
 constexpr int kPersistentFactor = 2;  // column groups per workgroup from which on workgroups walk
 
 
@@ -508,6 +506,10 @@ bool launch_independent_waves(const blkq4_gemm_args* a, int* status) {
   int rows_log2 = 0;
   while ((1 << rows_log2) < a->m) ++rows_log2;
   const size_t a_bytes = (((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023};
+  // measured break-even against workgroups that split K and walk (blocks along N gain more: their sixteen-wave
+  // kernel has no walking variant)
+  constexpr int kIndependentMinTiles = ROW ? 896 : 2000;
+  constexpr size_t kIndependentMaxRowBytes = (ROW ? 32 : 16) * 1024;
   if (a->n / 16 < kIndependentMinTiles || a_bytes > kIndependentMaxRowBytes ||
       (reinterpret_cast<uintptr_t>(a->c) & 7u) != 0) {
     return false;
