@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_PKG, "lib", "libms_blkq4gemm.so")
 
 EXPORTED_SYMBOLS = (
     "blkq4_fp16_gemm_sm80",
+    "blkq4_fp16_gemm_bias_sm80",
     "blkq4_fp16_quant_sm80",
     "blkq4_fp16_quant_size_sm80",
     "blkq4_fp16_repack_sm80",
@@ -49,6 +50,8 @@ def load() -> ctypes.CDLL:
     i64p = ctypes.POINTER(ctypes.c_int64)
     L.blkq4_fp16_gemm_sm80.argtypes = [i, b, i, i, i, vp, vp, sz, vp, sz, vp, sz, vp, sz, vp, sz, vp]
     L.blkq4_fp16_gemm_sm80.restype = i
+    L.blkq4_fp16_gemm_bias_sm80.argtypes = [i, b, i, i, i, vp, vp, sz, vp, sz, vp, sz, vp, sz, vp, sz, vp, sz, vp]
+    L.blkq4_fp16_gemm_bias_sm80.restype = i
     L.blkq4_fp16_quant_sm80.argtypes = [i, b, i, i, i, vp, vp, sz, vp, sz, vp, sz, vp, sz, vp]
     L.blkq4_fp16_quant_sm80.restype = i
     # `int64_t&` is a pointer at the ABI level
@@ -140,13 +143,19 @@ def quant(block_size: int, column_wise: bool, weights_nk, q_weights, q_scales, q
 
 
 def gemm(block_size: int, column_wise: bool, m: int, n: int, k: int, a, q_weights, q_scales, q_zp, out,
-         stream=None):
-    """``blkq4_fp16_gemm_sm80`` on device tensors."""
+         stream=None, bias=None):
+    """``blkq4_fp16_gemm_sm80`` on device tensors; with ``bias`` (fp16 ``[n]``) ``blkq4_fp16_gemm_bias_sm80``."""
     L = load()
     err = _ErrMsg(L)
-    rc = L.blkq4_fp16_gemm_sm80(block_size, column_wise, m, n, k, _stream_ptr(stream), _ptr(a), _nbytes(a),
-                                _ptr(q_weights), _nbytes(q_weights), _ptr(q_scales), _nbytes(q_scales),
-                                _ptr(q_zp), _nbytes(q_zp), _ptr(out), _nbytes(out), err.h)
+    if bias is None:
+        rc = L.blkq4_fp16_gemm_sm80(block_size, column_wise, m, n, k, _stream_ptr(stream), _ptr(a), _nbytes(a),
+                                    _ptr(q_weights), _nbytes(q_weights), _ptr(q_scales), _nbytes(q_scales),
+                                    _ptr(q_zp), _nbytes(q_zp), _ptr(out), _nbytes(out), err.h)
+    else:
+        rc = L.blkq4_fp16_gemm_bias_sm80(block_size, column_wise, m, n, k, _stream_ptr(stream), _ptr(a), _nbytes(a),
+                                         _ptr(q_weights), _nbytes(q_weights), _ptr(q_scales), _nbytes(q_scales),
+                                         _ptr(q_zp), _nbytes(q_zp), _ptr(bias), _nbytes(bias), _ptr(out),
+                                         _nbytes(out), err.h)
     _check(rc, err)
 
 

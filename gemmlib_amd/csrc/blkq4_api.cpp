@@ -167,14 +167,14 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_sm80(int block_size, bool column_wi
   return 0;
 }
 
-// reference: src/blkq4_f16_gemm_sm80.cu:319-429 and :38-153 (blkq4_gemm_sm80_T)
-extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wise_blocking, int m,
-                                                 int n, int k, void* stream, void const* act_ptr,
-                                                 size_t a_size, void const* weights_ptr,
-                                                 size_t weights_size, void const* scales_ptr,
-                                                 size_t scales_size, void const* offsets_ptr,
-                                                 size_t offsets_size, void* output_ptr,
-                                                 size_t output_size, void* err_msg_ptr) {
+namespace {
+
+// reference: src/blkq4_f16_gemm_sm80.cu:319-429 and :38-153 (blkq4_gemm_sm80_T); bias_ptr == nullptr or
+// bias_size == 0: no bias
+int gemm_entry(int block_size, bool column_wise_blocking, int m, int n, int k, void* stream, void const* act_ptr,
+               size_t a_size, void const* weights_ptr, size_t weights_size, void const* scales_ptr,
+               size_t scales_size, void const* offsets_ptr, size_t offsets_size, void const* bias_ptr,
+               size_t bias_size, void* output_ptr, size_t output_size, void* err_msg_ptr) {
   auto* err = static_cast<std::string*>(err_msg_ptr);
   if (!supported_block_size(block_size)) {
     set_error(err, "Unsupported block size: " + std::to_string(block_size));
@@ -217,6 +217,16 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
                        " expected: " + std::to_string(meta_elems));
     return -1;
   }
+  const bool has_bias = bias_ptr != nullptr && bias_size > 0;
+  if (has_bias && bias_size != N * 2) {
+    set_error(err, "Unexpected bias tensor size: " + std::to_string(bias_size) +
+                       " expected: " + std::to_string(N * 2));
+    return -1;
+  }
+  if (has_bias && !aligned16(bias_ptr)) {
+    set_error(err, "Kernel execution failed: Error Misaligned Operand");
+    return -1;
+  }
   // What the reference kernel's can_implement rejects
   // (src/mickey/cutlass_ext/q4gemm/kernel/quantb_gemm.h:172-255).
   if (!aligned16(act_ptr) || !aligned16(weights_ptr) || (k % 8) != 0) {
@@ -253,11 +263,41 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
   args.scales = scales_ptr;
   args.zero_points = has_offsets ? offsets_ptr : nullptr;
   args.c = output_ptr;
+  args.bias = has_bias ? bias_ptr : nullptr;
   args.stream = stream;
   // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
   const int code = streaming_kernel_takes(column_wise_blocking, m, n, k) ? blkq4_dev_skinny(&args) : blkq4_dev_gemm(&args);
   if (code) return device_failure(code, err);
   return 0;
+}
+
+}  // namespace
+
+extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wise_blocking, int m,
+                                                 int n, int k, void* stream, void const* act_ptr,
+                                                 size_t a_size, void const* weights_ptr,
+                                                 size_t weights_size, void const* scales_ptr,
+                                                 size_t scales_size, void const* offsets_ptr,
+                                                 size_t offsets_size, void* output_ptr,
+                                                 size_t output_size, void* err_msg_ptr) {
+  return gemm_entry(block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
+                    scales_ptr, scales_size, offsets_ptr, offsets_size, nullptr, 0, output_ptr, output_size,
+                    err_msg_ptr);
+}
+
+// the GEMM with the bias of the linear layer added in its epilogue (reference: python/ms_blkq4linear.py:26-27,
+// `output += self.bias` as a second kernel)
+extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_bias_sm80(int block_size, bool column_wise_blocking, int m,
+                                                      int n, int k, void* stream, void const* act_ptr,
+                                                      size_t a_size, void const* weights_ptr,
+                                                      size_t weights_size, void const* scales_ptr,
+                                                      size_t scales_size, void const* offsets_ptr,
+                                                      size_t offsets_size, void const* bias_ptr,
+                                                      size_t bias_size, void* output_ptr,
+                                                      size_t output_size, void* err_msg_ptr) {
+  return gemm_entry(block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
+                    scales_ptr, scales_size, offsets_ptr, offsets_size, bias_ptr, bias_size, output_ptr,
+                    output_size, err_msg_ptr);
 }
 
 extern "C" BLKQ4_EXPORT int blkq4_fp16_repack_sm80(int to_sm80, int rows, int columns, void* stream,

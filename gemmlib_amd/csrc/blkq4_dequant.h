@@ -121,4 +121,17 @@ __device__ __forceinline__ uint16_t float_to_half_bits(float f) {
   return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
 }
 
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
+}
+
+// c + bias the way an fp16 tensor library adds two fp16 tensors: in fp32, rounded to fp16 (the reference
+// module adds its bias to the fp16 output of the GEMM, python/ms_blkq4linear.py:26-27).
+__device__ __forceinline__ uint32_t add_bias_bits(uint32_t c, uint32_t bias) {
+  return float_to_half_bits(half_bits_to_float(c) + half_bits_to_float(bias));
+}
+__device__ __forceinline__ uint32_t add_bias_pair(uint32_t c, uint32_t bias) {
+  return add_bias_bits(c & 0xffffu, bias & 0xffffu) | (add_bias_bits(c >> 16, bias >> 16) << 16);
+}
+
 }  // namespace blkq4

@@ -55,6 +55,7 @@ typedef struct {
   const void* scales;       /* fp16 [K/bs][N]; column_wise = 0: packed [K][N/bs] order described above */
   const void* zero_points;  /* uint8, same shape and order as the scales, or NULL */
   void* c;                  /* fp16 [m][n] */
+  const void* bias;         /* fp16 [n] added to every row of c after its rounding to fp16, or NULL */
   void* stream;
 } blkq4_gemm_args;
 

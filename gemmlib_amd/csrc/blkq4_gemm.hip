@@ -104,7 +104,8 @@ template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW>
 __global__ __launch_bounds__(64 * (WM * WN + PW))
     __attribute__((amdgpu_waves_per_eu((WM * WN + PW) / 4, (WM * WN + PW) / 4))) void gemm_mfma_kernel(
         const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ S,
-        const uint8_t* __restrict__ Z, uint16_t* __restrict__ C, int M, int N, int K, int m_tiles) {
+        const uint8_t* __restrict__ Z, uint16_t* __restrict__ C, const uint16_t* __restrict__ bias, int M, int N,
+        int K, int m_tiles) {
   using St = Stage<BS, RT, NT, WM, WN, PW, ROW>;
   constexpr int kComputeWaves = WM * WN;
   static_assert(!ROW || St::kGroups % 2 == 0, "scale copies take two column groups at a time");
@@ -492,6 +493,9 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
     const uint32_t region = lds0 + (wm * WN + wn) * (32 * kPassTiles * kRowBytes);
     const int srow = lane / kChunks, chunk = lane % kChunks;
     const int col = nw0 + chunk * 8;
+    // the lane stores the same 8 columns of every row: their bias values are fetched once
+    uint4 bias8 = make_uint4(0, 0, 0, 0);
+    if (bias != nullptr && col < N) bias8 = *reinterpret_cast<const uint4*>(bias + col);
 #pragma unroll
     for (int r0 = 0; r0 < RT; r0 += kPassTiles) {
 #pragma unroll
@@ -511,7 +515,11 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
 #pragma unroll
       for (int it = 0; it < 32 * kPassTiles / kRowsPerStore; ++it) {
         const int row = it * kRowsPerStore + srow;  // inside the pass
-        const uint4 v = lds_read_16(region + srow * kRowBytes + chunk * 16, it * kRowsPerStore * kRowBytes);
+        uint4 v = lds_read_16(region + srow * kRowBytes + chunk * 16, it * kRowsPerStore * kRowBytes);
+        if (bias != nullptr) {
+          v = make_uint4(add_bias_pair(v.x, bias8.x), add_bias_pair(v.y, bias8.y), add_bias_pair(v.z, bias8.z),
+                         add_bias_pair(v.w, bias8.w));
+        }
         const int m = m0 + wm * (32 * RT) + r0 * 32 + row;
         if (m < M && col < N) *reinterpret_cast<uint4*>(C + static_cast<size_t>(m) * N + col) = v;
       }
@@ -529,8 +537,8 @@ int launch_one(const blkq4_gemm_args* a) {
   hipLaunchKernelGGL((gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW, ROW>), grid, dim3(64 * (WM * WN + PW)), 0,
                      static_cast<hipStream_t>(a->stream), static_cast<const uint8_t*>(a->a),
                      static_cast<const uint8_t*>(a->packed_w), static_cast<const uint8_t*>(a->scales),
-                     static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c), a->m, a->n,
-                     a->k, m_tiles);
+                     static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c),
+                     static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k, m_tiles);
   return static_cast<int>(hipGetLastError());
 }
 

@@ -76,7 +76,8 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
                                                                const uint4* __restrict__ W,
                                                                const uint16_t* __restrict__ S,
                                                                const uint8_t* __restrict__ Z,
-                                                               uint16_t* __restrict__ C, int M_total, int N,
+                                                               uint16_t* __restrict__ C,
+                                                               const uint16_t* __restrict__ bias, int M_total, int N,
                                                                int K, int rows_log2, int row_groups,
                                                                int cg_stride, uint32_t red_offset) {
   constexpr int kMeta = Slot<BS, NT, MT, AM, ROW>::kMeta;
@@ -254,8 +255,13 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
           const int tile = (cgx * kTileWaves + wt) * NT + t;
           const int row = 16 * mt + nl;
           if (row < M && tile < tiles) {
-            const uint32_t lo = float_to_half_bits(acc[t][mt][0]) | (static_cast<uint32_t>(float_to_half_bits(acc[t][mt][1])) << 16);
-            const uint32_t hi = float_to_half_bits(acc[t][mt][2]) | (static_cast<uint32_t>(float_to_half_bits(acc[t][mt][3])) << 16);
+            uint32_t lo = float_to_half_bits(acc[t][mt][0]) | (static_cast<uint32_t>(float_to_half_bits(acc[t][mt][1])) << 16);
+            uint32_t hi = float_to_half_bits(acc[t][mt][2]) | (static_cast<uint32_t>(float_to_half_bits(acc[t][mt][3])) << 16);
+            if (bias != nullptr) {
+              const uint2 b = *reinterpret_cast<const uint2*>(bias + tile * 16 + 4 * g);
+              lo = add_bias_pair(lo, b.x);
+              hi = add_bias_pair(hi, b.y);
+            }
             *reinterpret_cast<uint2*>(C + static_cast<size_t>(row) * N + tile * 16 + 4 * g) = make_uint2(lo, hi);
           }
           acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -281,7 +287,10 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       const int t = v / (MT * 256), mt = (v >> 8) % MT, L = (v >> 2) & 63, e = v & 3;
       const int row = 16 * mt + (L & 15);
       if (row < M && cgx * NT + t < tiles) {
-        C[static_cast<size_t>(row) * N + cgx * (16 * NT) + 16 * t + 4 * (L >> 4) + e] = float_to_half_bits(r);
+        const int col = cgx * (16 * NT) + 16 * t + 4 * (L >> 4) + e;
+        uint32_t h = float_to_half_bits(r);
+        if (bias != nullptr) h = add_bias_bits(h, bias[col]);
+        C[static_cast<size_t>(row) * N + col] = static_cast<uint16_t>(h);
       }
     }
   };
@@ -478,7 +487,8 @@ int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * kWaves), lds_bytes, static_cast<hipStream_t>(a->stream),
                        static_cast<const uint16_t*>(a->a), static_cast<const uint4*>(a->packed_w),
                        static_cast<const uint16_t*>(a->scales), static_cast<const uint8_t*>(a->zero_points),
-                       static_cast<uint16_t*>(a->c), a->m, a->n, a->k, rows_log2, row_groups, cg_stride,
+                       static_cast<uint16_t*>(a->c), static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k,
+                       rows_log2, row_groups, cg_stride,
                        static_cast<uint32_t>(red_offset));
     return static_cast<int>(hipGetLastError());
   };

@@ -2,7 +2,7 @@
 // three C entry points.  Same Python surface as the reference extension
 // (reference: python/ms_blkq4linear_ext/ms_blkq4linear.cpp:13-123):
 //   quant(block_size, col_wise, has_offsets, weights) -> [q_weights(uint8), q_scales(fp16), q_zp(uint8)]
-//   forward(block_size, col_wise, in_features, out_features, input, q_weights, q_scales, q_zp) -> Tensor
+//   forward(block_size, col_wise, in_features, out_features, input, q_weights, q_scales, q_zp, bias=None) -> Tensor
 // Differences on purpose: kernels run on torch's current stream instead of the default stream, and a
 // scale-only quantization returns an empty uint8 tensor for q_zp (the reference returns an undefined
 // tensor that its own forward() cannot take).
@@ -60,7 +60,8 @@ std::vector<torch::Tensor> blkq4linear_quant(int64_t block_size, bool col_wise, 
 
 torch::Tensor blkq4linear_forward(int64_t block_size, bool col_wise, int64_t in_features,
                                   int64_t out_features, torch::Tensor input, torch::Tensor q_weights,
-                                  torch::Tensor q_scales, torch::Tensor q_zp) {
+                                  torch::Tensor q_scales, torch::Tensor q_zp,
+                                  const c10::optional<torch::Tensor>& bias) {
   TORCH_CHECK(input.scalar_type() == torch::kFloat16, "blkq4linear_forward only supports float16 inputs");
   TORCH_CHECK(input.dim() == 2 && input.size(1) == in_features,
               "Activation shape is not compatible with the weights");
@@ -79,13 +80,28 @@ torch::Tensor blkq4linear_forward(int64_t block_size, bool col_wise, int64_t in_
     zp_ptr = q_zp.data_ptr();
     zp_bytes = static_cast<size_t>(q_zp.numel());
   }
+  // the bias is added in the GEMM's epilogue (the reference module adds it with a second kernel,
+  // python/ms_blkq4linear.py:26-27); a bias that is not 16-byte aligned is copied first
+  torch::Tensor bias_t;
+  const void* bias_ptr = nullptr;
+  size_t bias_bytes = 0;
+  if (bias.has_value() && bias->defined() && bias->numel() > 0) {
+    TORCH_CHECK(bias->scalar_type() == torch::kFloat16 && bias->dim() == 1 && bias->size(0) == out_features,
+                "blkq4linear_forward: the bias must be a float16 tensor of out_features elements");
+    TORCH_CHECK(bias->device() == dev, "blkq4linear_forward requires all tensors on the same device");
+    bias_t = bias->contiguous();
+    if ((reinterpret_cast<uintptr_t>(bias_t.data_ptr()) & 15u) != 0) bias_t = bias_t.clone();
+    bias_ptr = bias_t.data_ptr();
+    bias_bytes = bias_t.numel() * kHalfBytes;
+  }
   std::string err;
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(dev.index()).stream();
-  const int rc = blkq4_fp16_gemm_sm80(
+  const int rc = blkq4_fp16_gemm_bias_sm80(
       static_cast<int>(block_size), col_wise, static_cast<int>(input.size(0)), static_cast<int>(out_features),
       static_cast<int>(in_features), stream, input.data_ptr(), input.numel() * kHalfBytes,
       q_weights.data_ptr(), static_cast<size_t>(q_weights.numel()), q_scales.data_ptr(),
-      q_scales.numel() * kHalfBytes, zp_ptr, zp_bytes, output.data_ptr(), output.numel() * kHalfBytes, &err);
+      q_scales.numel() * kHalfBytes, zp_ptr, zp_bytes, bias_ptr, bias_bytes, output.data_ptr(),
+      output.numel() * kHalfBytes, &err);
   TORCH_CHECK(rc == 0, err);
   return output;
 }
@@ -94,5 +110,8 @@ torch::Tensor blkq4linear_forward(int64_t block_size, bool col_wise, int64_t in_
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("quant", &blkq4linear_quant, "Quantize float 16 weights");
-  m.def("forward", &blkq4linear_forward, "Forward pass for block quantized linear layer");
+  m.def("forward", &blkq4linear_forward, "Forward pass for block quantized linear layer", pybind11::arg("block_size"),
+        pybind11::arg("col_wise"), pybind11::arg("in_features"), pybind11::arg("out_features"),
+        pybind11::arg("input"), pybind11::arg("q_weights"), pybind11::arg("q_scales"), pybind11::arg("q_zp"),
+        pybind11::arg("bias") = pybind11::none());
 }

@@ -3,7 +3,9 @@
 Same constructor, attributes and ``forward`` as the reference module
 (reference: python/ms_blkq4linear.py:10-28): ``weights`` is the fp16 ``[out_features, in_features]``
 tensor on the GPU, ``scale_only`` selects the symmetric quantizer (no zero-points), the packed
-tensors are reachable as ``q_weights`` / ``q_scales`` / ``q_zp`` and the bias is added in place.
+tensors are reachable as ``q_weights`` / ``q_scales`` / ``q_zp``.  The bias is added by the GEMM's epilogue
+with the same two roundings as the reference's in-place ``output += self.bias`` (python/ms_blkq4linear.py:26-27),
+so the result is bit for bit the same without a second kernel.
 All device work happens in the HIP library behind ``ms_blkq4linear_ext``; there is no fallback.
 
 Beyond the reference (which keeps the packed tensors as plain attributes, so ``state_dict()`` loses
@@ -72,9 +74,7 @@ class BlkQ4Linear(nn.Module):
         lead = input.shape[:-1]
         x = input if input.dim() == 2 else input.reshape(-1, input.shape[-1])
         output = ms_blkq4linear_ext.forward(self.block_size, self.col_wise, self.in_features, self.out_features,
-                                            x, self.q_weights, self.q_scales, self.q_zp)
-        if self.bias is not None:
-            output += self.bias
+                                            x, self.q_weights, self.q_scales, self.q_zp, self.bias)
         return output if input.dim() == 2 else output.reshape(*lead, self.out_features)
 
     def extra_repr(self):

@@ -50,6 +50,29 @@ int blkq4_fp16_gemm_sm80(
   void* error_message);
 
 /**
+ * The GEMM above with the bias of the linear layer added in its epilogue: every row of C gets
+ * bias[0..n) (fp16) added AFTER the sum has been rounded to fp16, in fp32 and rounded to fp16 again,
+ * which is bit for bit what the reference module's `output += self.bias` computes with a second
+ * kernel (reference: python/ms_blkq4linear.py:26-27).  bias_size = n*2, bias 16-byte aligned;
+ * bias_ptr == nullptr or bias_size == 0 means no bias (then identical to blkq4_fp16_gemm_sm80).
+ *
+ * No counterpart in the reference's C API (its module adds the bias itself); every other argument,
+ * check and message as in blkq4_fp16_gemm_sm80.
+ */
+int blkq4_fp16_gemm_bias_sm80(
+  int block_size,
+  bool column_wise_blocking,
+  int m, int n, int k,
+  void* stream,
+  void const* act_ptr, size_t a_size,
+  void const* weights_ptr, size_t weights_size,
+  void const* scales_ptr, size_t scales_size,
+  void const* offsets_ptr, size_t offsets_size,
+  void const* bias_ptr, size_t bias_size,
+  void* output_ptr, size_t output_size,
+  void* error_message);
+
+/**
  * Quantize an fp16 weight matrix blockwise to 4 bits and pack it for the GEMM above.
  * `weights` holds element (row r, column c) at weights[r + c * leadingDimension] (rows = in_features,
  * columns = out_features, i.e. a torch [out, in] contiguous tensor with leadingDimension = in).

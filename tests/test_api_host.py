@@ -78,12 +78,12 @@ def _buf(nbytes, address=0x1000):
     return RawBuffer(address, nbytes)
 
 
-def _gemm(capi, bs=32, col=True, m=4, n=64, k=64, a=None, w=None, s=None, z=None, c=None):
+def _gemm(capi, bs=32, col=True, m=4, n=64, k=64, a=None, w=None, s=None, z=None, c=None, bias=None):
     a = _buf(m * k * 2) if a is None else a
     w = _buf(k * n // 2) if w is None else w
     s = _buf((k // bs) * n * 2) if s is None else s
     c = _buf(m * n * 2) if c is None else c
-    capi.gemm(bs, col, m, n, k, a, w, s, z, c, stream=0)
+    capi.gemm(bs, col, m, n, k, a, w, s, z, c, stream=0, bias=bias)
 
 
 @pytest.mark.parametrize("kwargs,message", [
@@ -99,6 +99,11 @@ def _gemm(capi, bs=32, col=True, m=4, n=64, k=64, a=None, w=None, s=None, z=None
      "Kernel execution failed: Error Invalid Problem"),
     (dict(a=_buf(512, address=0x1002)), "Kernel execution failed: Error Misaligned Operand"),
     (dict(c=_buf(512, address=0x1008)), "Kernel execution failed: Error Misaligned Operand"),
+    # the entry point with a bias: its size and alignment, and the checks of the plain one in the same order
+    (dict(bias=_buf(126)), "Unexpected bias tensor size: 126 expected: 128"),
+    (dict(bias=_buf(128, address=0x1008)), "Kernel execution failed: Error Misaligned Operand"),
+    (dict(bias=_buf(128), c=_buf(8)), "Unexpected output tensor size: 8 expected: 512"),
+    (dict(bias=_buf(128), bs=8), "Unsupported block size: 8"),
     # blocks along N: the scales are fetched 16 bytes at a time; n must be a multiple of the block size
     (dict(col=False, s=_buf(64 * 2 * 2, address=0x1004)), "Kernel execution failed: Error Misaligned Operand"),
     (dict(col=False, bs=64, n=96, w=_buf(64 * 96 // 2), s=_buf(64 * 1 * 2), c=_buf(4 * 96 * 2)),

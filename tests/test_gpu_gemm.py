@@ -179,6 +179,35 @@ def test_weights_repacked_from_reference_order(oracle, capi, device):
     assert np.array_equal(got.view(np.uint16), oracle.gemm(a, kat["weights"]).view(np.uint16))
 
 
+# (block_size, has_offsets, column_wise, m, n, k): every kernel and epilogue that stores outputs: streaming kernel
+# with sums across waves (M = 1, 16), with row groups (M = 64), with waves that keep whole sums (wide N), and
+# the tile kernel's three shapes
+BIAS_CASES = [
+    (64, False, True, 1, 4096, 512), (32, True, True, 16, 1056, 576), (16, True, True, 64, 352, 256),
+    (64, False, True, 2, 32000, 256), (32, True, False, 3, 16384, 128), (64, True, True, 300, 4128, 192),
+    (32, True, True, 1100, 4160, 128), (16, True, True, 4096, 4096, 64), (64, True, False, 1200, 1088, 192),
+]
+
+
+@pytest.mark.parametrize("bs,has_offsets,col,m,n,k", BIAS_CASES)
+def test_bias_in_the_epilogue_equals_a_separate_add(oracle, capi, device, bs, has_offsets, col, m, n, k):
+    """blkq4_fp16_gemm_bias_sm80 == blkq4_fp16_gemm_sm80 followed by the tensor library's in-place fp16 add
+    (what the reference module does, python/ms_blkq4linear.py:26-27), bit for bit."""
+    a, w = gaussian_problem(m + n + k, m, n, k)
+    g = torch.Generator(device="cpu").manual_seed(n)
+    bias = (torch.randn(n, generator=g) * 0.5).to(torch.float16).to(device)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, w, has_offsets, column_wise=col)
+    a_dev = to_dev(a, device)
+    plain = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+    fused = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+    capi.gemm(bs, col, m, n, k, a_dev, q_w, q_s, q_zp, plain)
+    capi.gemm(bs, col, m, n, k, a_dev, q_w, q_s, q_zp, fused, bias=bias)
+    torch.cuda.synchronize()
+    plain += bias
+    assert not torch.isnan(fused).any()
+    assert torch.equal(fused.view(torch.int16), plain.view(torch.int16))
+
+
 def test_non_default_stream(oracle, capi, device):
     a, w = gaussian_problem(5, 8, 256, 256)
     q_w, q_s, q_zp = quantize_on_gpu(capi, device, 64, w, True)
