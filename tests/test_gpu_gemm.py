@@ -85,7 +85,7 @@ LONG_K_CASES = [
 # several column groups (rows whole in LDS, rows staged per slice, row groups of 32)
 VERY_WIDE_CASES = [
     (64, False, 1, 32000, 4096), (32, True, 2, 32032, 4032), (16, True, 4, 32768, 320), (64, True, 1, 32000, 8192),
-    (64, False, 1, 14336, 4096), (32, True, 2, 16416, 4160),
+    (64, False, 1, 14336, 4096), (32, True, 2, 16416, 4160), (32, False, 16, 32032, 256), (16, True, 9, 32000, 448),
     (64, True, 8, 32800, 4096), (32, True, 16, 16416, 8256), (32, True, 96, 5440, 4160), (16, False, 12, 28672, 1088),
 ]
 

@@ -50,6 +50,7 @@ TILE_CASES = [
 # walk over several column groups
 VERY_WIDE_CASES = [
     (64, False, 1, 14336, 4096), (32, True, 2, 16384, 2112), (16, True, 8, 28672, 1088), (64, True, 16, 16384, 8256),
+    (32, True, 16, 14336, 960), (64, False, 5, 32000, 320),
 ]
 
 
