@@ -1,0 +1,75 @@
+"""GPU parity of the GEMM on seeded random shapes, through the C ABI, against the oracle.
+
+The shapes are drawn so that every way the library splits the work is hit with ragged edges: K that ends
+inside a 128-deep slice, column tile counts that the column groups do not divide, row counts around the
+row-group and kernel switches, very wide N (waves with a column tile of their own, workgroups that walk over
+several column groups), both blockings, with and without zero-points and bias.  Bar: max relative error
+<= 1e-2 on Gaussian data, where the error of an output is measured against max(|ref|, 1e-3 * max|ref|).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import max_rel_err, quantize_on_gpu, to_dev, to_np
+from test_gpu_gemm import gaussian_problem
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = 1e-2
+
+
+def draw_cases():
+    rng = np.random.default_rng(20240229)
+    cases = []
+    for i in range(48):
+        bs = int(rng.choice([16, 32, 64]))
+        col = bool(rng.integers(0, 2))
+        zp = bool(rng.integers(0, 2))
+        band = i % 4
+        if band == 0:    # few rows, very wide
+            m = int(rng.integers(1, 17))
+            n = int(rng.integers(14336 // 64, 40000 // 64)) * 64
+            k = int(rng.integers(1, 24)) * 64
+        elif band == 1:  # few rows, moderately wide, long K
+            m = int(rng.integers(1, 17))
+            n = int(rng.integers(1, 200)) * 64
+            k = int(rng.integers(8, 140)) * 64
+        elif band == 2:  # row groups
+            m = int(rng.integers(17, 400))
+            n = int(rng.integers(1, 150)) * 64
+            k = int(rng.integers(1, 40)) * 64
+        else:            # tile kernel
+            m = int(rng.integers(400, 2500))
+            n = int(rng.integers(1, 70)) * 64
+            k = int(rng.integers(1, 12)) * 64
+        if col and rng.integers(0, 2):
+            n += 32  # blocks along K allow any multiple of 32
+        cases.append((bs, zp, col, m, n, k, bool(rng.integers(0, 2))))
+    return cases
+
+
+@pytest.mark.parametrize("bs,has_offsets,col,m,n,k,with_bias", draw_cases())
+def test_random_shape(oracle, capi, device, bs, has_offsets, col, m, n, k, with_bias):
+    a, w = gaussian_problem(m * 7 + n * 3 + k, m, n, k)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, w, has_offsets, column_wise=col)
+    a_dev = to_dev(a, device)
+    out = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+    capi.gemm(bs, col, m, n, k, a_dev, q_w, q_s, q_zp, out)
+    torch.cuda.synchronize()
+    got = to_np(out)
+    assert not np.isnan(got).any()
+    canon, s, z = oracle.quantize(bs, col, w, has_offsets)
+    rows = np.arange(m) if m * n * k <= 3e9 else np.unique(np.concatenate([[0, m - 1], np.arange(0, m, max(1, m // 64))]))
+    ref = oracle.gemm(np.ascontiguousarray(a[rows]), oracle.dequantize(bs, col, canon, s, z))
+    assert max_rel_err(got[rows], ref) <= TOLERANCE
+    if with_bias:
+        # the fused bias against the separate add, bit for bit (an error bound against the oracle would measure
+        # the cancellation between sum and bias, not the kernel)
+        g = torch.Generator(device="cpu").manual_seed(n + k)
+        bias = (torch.randn(n, generator=g) * 0.25).to(torch.float16).to(device)
+        fused = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+        capi.gemm(bs, col, m, n, k, a_dev, q_w, q_s, q_zp, fused, bias=bias)
+        torch.cuda.synchronize()
+        out += bias
+        assert torch.equal(fused.view(torch.int16), out.view(torch.int16))
