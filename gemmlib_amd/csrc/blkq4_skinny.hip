@@ -10,7 +10,7 @@
 //     every wave the chip holds (and few rows), the waves do not split K: each has column tiles of its own,
 //     streams all of K, and stores its sums itself: no barrier after the rows have arrived;
 //   - a wave keeps the weight units, scales and zero-points of DEPTH slices in flight and refills a
-//     slot as soon as it has consumed it (out-of-range slices wrap around to valid units and are
+//     slot as soon as it has consumed it (a slot past the end asks for valid units once more and is
 //     multiplied by a zero scale, so the loop has no divergent loads);
 //   - the activation rows are copied into LDS by asynchronous global_load_lds copies, laid out per 32-deep
 //     unit as [unit][row][64 bytes] (16-byte chunks XOR-swizzled with bits 2..3 of the row so that a
@@ -35,6 +35,8 @@
 
 #include <stdint.h>
 
+#include <atomic>
+
 #include "blkq4_dequant.h"
 #include "blkq4_device.h"
 #include "blkq4_gemm_common.h"
@@ -57,7 +59,6 @@ struct Slot {
   // the meta data (two 16-row groups of 32 + 16 bytes)
   uint4 rs[ROW ? NT : 1][4];
   uint4 rz[ROW ? NT : 1][2];
-
 };
 
 // kWaves: waves of the workgroup.  kSplit: how many of them split K: all (kSplit = kWaves; their partial tiles
@@ -86,7 +87,8 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   constexpr int kLoads = ROW ? NT * (1 + 4 + (HAS_ZP ? 2 : 0)) : NT * (1 + kMeta * (HAS_ZP ? 2 : 1));
   constexpr int kSlotRows = 16 * MT;                           // kRowsPerSlotInLds: rows staged per slot
   constexpr int kSlotBytes = kSlotRows * 256;
-  // the partial tiles of the final reduction reuse the LDS of the activation rows
+  // the partial tiles of the sums across waves reuse the LDS of the activation rows (red_offset = 0) or, when
+  // the workgroup goes on to another column group and needs the rows again, lie behind them
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   float* red = reinterpret_cast<float*>(smem + red_offset);
   const uint8_t* a_lds = smem;
@@ -232,7 +234,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     }                                                                                          \
   }
   // A wave's local slices are li = 0 .. my_slices - 1 (slice ws + kSplit * li), taken DEPTH at a time; the
-  // slots past my_slices in the last round wrap around and are zeroed.
+  // slots past my_slices in the last round ask for the last slice once more and are zeroed.
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) BLKQ4_LOAD_SLOT(slot[d], d, cg, ws + kSplit * d, -1);
   if (A_LDS) {
@@ -444,7 +446,21 @@ void choose_shape(int m, int n, int* nt, int* depth) {
   *depth = (*nt == 1 && tiles <= 2 * kComputeUnits) ? 8 : 4;
 }
 
-// One kernel instantiation: raises its dynamic-LDS limit once, then launches `row_groups` row groups of
+// Raises a kernel's dynamic-LDS limit, once per kernel and device (the attribute belongs to the device's copy
+// of the code).
+template <class Kernel>
+hipError_t raise_lds_limit(Kernel* kernel) {
+  static std::atomic<uint64_t> done{0};  // one flag per device index below 64, one set of flags per kernel
+  int device = 0;
+  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
+  if (device < 64 && ((done.load(std::memory_order_acquire) >> device) & 1u) != 0) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
+  if (e == hipSuccess && device < 64) done.fetch_or(uint64_t{1} << device, std::memory_order_release);
+  return e;
+}
+
+// One kernel instantiation: raises its dynamic-LDS limit, then launches `row_groups` row groups of
 // 16 * MT rows each.
 template <int BS, bool HAS_ZP, bool ROW, int DEPTH, int NT, int MT, int kWaves, int AM, int kSplit = kWaves>
 int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
@@ -494,17 +510,13 @@ int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
   };
   if (refill) {
     auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, true, kSplit>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
-    return launch(kernel, attr);
+    return launch(kernel, raise_lds_limit(kernel));
   }
   if constexpr (kSplit == 1) {
     return static_cast<int>(hipErrorInvalidValue);  // not reached
   } else {
     auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, false, kSplit>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
-    return launch(kernel, attr);
+    return launch(kernel, raise_lds_limit(kernel));
   }
 }
 
