@@ -574,7 +574,7 @@ int launch_shape(const blkq4_gemm_args* a) {
   if (a->m > 16) {
     // Every workgroup fetches the 32 rows of its group for all of K, so wide workgroups (more column tiles)
     // mean less activation traffic; but there should be a workgroup for every compute unit.
-      const int row_groups = (a->m + 31) / 32;
+    const int row_groups = (a->m + 31) / 32;
     const long tiles = static_cast<long>(a->n / 16) * row_groups;
     if (tiles >= 4 * kComputeUnits) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 4>(a, row_groups);
     if (tiles >= 2 * kComputeUnits) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 2>(a, row_groups);
