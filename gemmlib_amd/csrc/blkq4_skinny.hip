@@ -604,6 +604,7 @@ int launch_skinny(const blkq4_gemm_args* a) {
 
 extern "C" int blkq4_dev_skinny(const blkq4_gemm_args* a) {
   if (a->m < 1 || a->m > kStreamingMaxRows || (a->n % 16) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
+  if (a->n > (1 << 26)) return static_cast<int>(hipErrorInvalidValue);  // a lane's offset inside a slice (up to 8 n rows of 16 bytes) is 32 bits wide
   if (!a->column_wise) {
     // blocks along N: a 16-column tile lies inside one block, and the meta data are fetched 16 bytes at a time
     if ((a->n % a->block_size) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 15u) != 0 ||
