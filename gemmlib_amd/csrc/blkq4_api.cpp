@@ -23,20 +23,34 @@ inline void set_error(std::string* err, std::string&& text) {
 // f16_gemm_sm80.h:63-72).  Here the weight-streaming kernel keeps going, in row groups of 32, for as long as
 // it is expected to be faster than the tile kernel, whose grid cannot fill the chip when m is small.
 // Both estimates are fits to measurements on MI355X: the streaming kernel's time grows with
-// row groups x n x k (2.8 us per row group at n = k = 4096); the tile kernel runs its k / 64 steps once per
-// round of 256 workgroups, 0.64 us a step with 128 x 256 tiles and 0.42 us with the 128 x 128 tiles it uses
-// when those cover the problem in one round.
+// row groups x n x k (2.8 us per row group at n = k = 4096) and, once it has more workgroups than compute
+// units, with whole rounds of them; the tile kernel runs its k / 64 steps once per round of 256 workgroups,
+// 0.64 us a step with 128 x 256 tiles, 0.42 us with the 128 x 128 tiles it uses when those cover the problem
+// in one round and 0.32 to 0.43 us (96 to 256 workgroups) with 64 x 128 tiles when even those do.
 inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k) {
   if (m <= 32) return true;
   if (m > 1024) return false;
-  const double row_groups = (m + 31) / 32;
+  const long row_groups = (m + 31) / 32;
   // blocks along N: the streaming kernel converts with 23 instead of 13 instructions per 8 weights
-  const double streaming_us = (column_wise ? 2.8 : 5.6) * row_groups * (static_cast<double>(n) / 4096.0) *
-                              (static_cast<double>(k) / 4096.0);
+  double streaming_us = (column_wise ? 2.8 : 5.6) * static_cast<double>(row_groups) * (static_cast<double>(n) / 4096.0) *
+                        (static_cast<double>(k) / 4096.0);
+  {
+    // its workgroups take 4, 2 or 1 column tiles of 16 (blocks along N: 1), as blkq4_skinny.hip chooses them
+    const long tiles = static_cast<long>(n / 16) * row_groups;
+    const long per_group = !column_wise ? 1 : tiles >= 1024 ? 4 : tiles >= 512 ? 2 : 1;
+    const long streaming_groups = row_groups * ((n / 16 + per_group - 1) / per_group);
+    if (streaming_groups > 256) {
+      streaming_us *= static_cast<double>((streaming_groups + 255) / 256) / (static_cast<double>(streaming_groups) / 256.0);
+    }
+  }
+  const long smallest_tiles = static_cast<long>((m + 63) / 64) * ((n + 127) / 128);
   const long small_tiles = static_cast<long>((m + 127) / 128) * ((n + 127) / 128);
   const long workgroups = static_cast<long>((m + 127) / 128) * ((n + 255) / 256);
-  const double tile_us = (small_tiles <= 256) ? (k / 64) * 0.42
-                                              : static_cast<double>((workgroups + 255) / 256) * (k / 64) * 0.64;
+  // (up to 64 rows the tile kernel has 64 x 256 tiles only: few workgroups, 0.55 us a step)
+  const double tile_us = (m <= 64) ? (k / 64) * 0.55
+                         : (smallest_tiles <= 256) ? (k / 64) * (0.25 + 0.0007 * static_cast<double>(smallest_tiles))
+                         : (small_tiles <= 256) ? (k / 64) * 0.42
+                                                : static_cast<double>((workgroups + 255) / 256) * (k / 64) * 0.64;
   return streaming_us < tile_us;
 }
 
