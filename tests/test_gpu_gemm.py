@@ -64,6 +64,8 @@ EDGE_CASES = [
 # tile count fills the chip (258 tiles: 2; 514: 3 with a ragged last workgroup; 1792: 1)
 # shapes with at least 256 tiles of 256 x 256, which take the kernel variant with 256-row waves
 LARGE_TILE_CASES = [(64, True, 4096, 4096, 128), (16, True, 4000, 4128, 64), (32, False, 4096, 4096, 192)]
+# shapes that 64 x 128 tiles cover in one round of workgroups (and the streaming kernel is not expected to beat)
+SMALL_TILE_CASES = [(64, True, 300, 4128, 192), (16, True, 500, 2080, 128), (32, False, 257, 4096, 64)]
 WIDE_SKINNY_CASES = [
     (16, True, 12, 4128, 128), (32, True, 8, 8224, 128), (64, False, 3, 8224, 192), (32, False, 5, 28672, 64),
 ]
@@ -90,7 +92,7 @@ VERY_WIDE_CASES = [
 ]
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + LONG_K_CASES + VERY_WIDE_CASES)
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + SMALL_TILE_CASES + LONG_K_CASES + VERY_WIDE_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
 

@@ -37,12 +37,12 @@ EDGE_CASES = [
 ]
 
 
-# the tile kernel's three shapes (128 x 128, 128 x 256 and 256 x 256 tiles) with every block size, N that ends
+# the tile kernel's four shapes (64 x 128, 128 x 128, 128 x 256 and 256 x 256 tiles) with every block size, N that ends
 # inside a tile, and row counts just past what the streaming kernel takes
 TILE_CASES = [
     (16, True, 400, 672, 576), (32, True, 1000, 4128, 128), (64, False, 1100, 4160, 192), (64, True, 640, 4160, 192),
     (16, True, 4096, 4096, 128), (32, False, 4000, 4128, 64), (64, True, 4096, 4096, 192), (16, False, 4090, 4128, 64),
-    (32, True, 160, 96, 8256), (16, False, 130, 2080, 128),
+    (32, True, 160, 96, 8256), (16, False, 130, 2080, 128), (32, True, 400, 2112, 128), (64, False, 300, 4160, 192),
 ]
 
 
