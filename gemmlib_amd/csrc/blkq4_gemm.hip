@@ -562,6 +562,8 @@ int launch_rt(const blkq4_gemm_args* a) {
     return launch_one<BS, HAS_ZP, 4, 2, 1, 4, 4, true>(a);
   }
   // rows per workgroup: no more than the problem has
+  // (32 rows: 32 x 128 tiles when there are enough of them to fill the chip, else 32 x 256 with eight waves)
+  if (a->m <= 32 && a->n / 128 >= 224) return launch_one<BS, HAS_ZP, 1, 1, 1, 4, 4>(a);
   if (a->m <= 32) return launch_one<BS, HAS_ZP, 1, 1, 1, 8, 0>(a);
   if (a->m <= 64) return launch_one<BS, HAS_ZP, 2, 1, 1, 8, 0>(a);
 #ifdef BLKQ4_GEMM_SHAPE

@@ -66,6 +66,9 @@ EDGE_CASES = [
 LARGE_TILE_CASES = [(64, True, 4096, 4096, 128), (16, True, 4000, 4128, 64), (32, False, 4096, 4096, 192)]
 # shapes that 64 x 128 tiles cover in one round of workgroups (and the streaming kernel is not expected to beat)
 SMALL_TILE_CASES = [(64, True, 300, 4128, 192), (16, True, 500, 2080, 128), (32, False, 257, 4096, 64)]
+# up to 32 rows, K too long for the streaming kernel to keep the rows in LDS, N wide enough for 32 x 128 tiles to
+# fill the chip: the tile kernel takes these
+WIDE_TILE32_CASES = [(64, True, 16, 28672, 5184), (32, True, 9, 28704, 5248), (16, False, 32, 28672, 2624), (64, False, 20, 28672, 2688)]
 WIDE_SKINNY_CASES = [
     (16, True, 12, 4128, 128), (32, True, 8, 8224, 128), (64, False, 3, 8224, 192), (32, False, 5, 28672, 64),
 ]
@@ -92,7 +95,7 @@ VERY_WIDE_CASES = [
 ]
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + SMALL_TILE_CASES + LONG_K_CASES + VERY_WIDE_CASES)
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + SMALL_TILE_CASES + WIDE_TILE32_CASES + LONG_K_CASES + VERY_WIDE_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
 
