@@ -28,12 +28,13 @@ inline void set_error(std::string* err, std::string&& text) {
 // 0.64 us a step with 128 x 256 tiles, 0.42 us with the 128 x 128 tiles it uses when those cover the problem
 // in one round and 0.32 to 0.43 us (96 to 256 workgroups) with 64 x 128 tiles when even those do.
 inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k) {
+  if (m <= 16) return true;
   if (m <= 32) {
-    // Up to 32 rows the streaming kernel wins unless it cannot keep the rows in LDS for all of K (it then
-    // fetches them again for every column group) and the problem is wide enough for 32 x 128 tiles to fill the
-    // chip: M = 16, K = 8192, N = 28672 takes 57.6 us streaming and 44.7 us in tiles.
-    const long rows = (m > 16) ? 32 : (m > 8) ? 16 : (m > 4) ? 8 : (m > 2) ? 4 : m;
-    const bool rows_fit = rows * static_cast<long>(k) * 2 <= 160 * 1024;
+    // 17 to 32 rows: the streaming kernel wins unless it cannot keep the rows in LDS for all of K (it then
+    // fetches them again for every column group) and the problem is wide enough for the tile kernel's 32-row
+    // tiles to fill the chip: M = 32, K = 4096, N = 28672 takes 27.3 us streaming and 23.1 us in tiles, with
+    // N = 65536 53.7 and 39.5 us.
+    const bool rows_fit = 32L * k * 2 <= 160 * 1024;
     return !column_wise || rows_fit || n / 128 < 224;
   }
   if (m > 1024) return false;

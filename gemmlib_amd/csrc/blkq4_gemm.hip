@@ -562,9 +562,12 @@ int launch_rt(const blkq4_gemm_args* a) {
     return launch_one<BS, HAS_ZP, 4, 2, 1, 4, 4, true>(a);
   }
   // rows per workgroup: no more than the problem has
-  // (32 rows: 32 x 128 tiles when there are enough of them to fill the chip, else 32 x 256 with eight waves)
-  if (a->m <= 32 && a->n / 128 >= 224) return launch_one<BS, HAS_ZP, 1, 1, 1, 4, 4>(a);
+  // (up to 64 rows: 128 columns with four waves and four producer waves when such tiles fill the chip in one
+  // round, else 256 columns with eight waves; M = 64, K = 4096, N = 28672: 34.7 against 26.3 us)
+  const bool one_round_of_128 = a->n / 128 >= 224 && a->n / 128 <= kComputeUnits;
+  if (a->m <= 32 && one_round_of_128) return launch_one<BS, HAS_ZP, 1, 1, 1, 4, 4>(a);
   if (a->m <= 32) return launch_one<BS, HAS_ZP, 1, 1, 1, 8, 0>(a);
+  if (a->m <= 64 && one_round_of_128) return launch_one<BS, HAS_ZP, 2, 1, 1, 4, 4>(a);
   if (a->m <= 64) return launch_one<BS, HAS_ZP, 2, 1, 1, 8, 0>(a);
 #ifdef BLKQ4_GEMM_SHAPE
   return launch_one<BS, HAS_ZP, BLKQ4_GEMM_SHAPE>(a);

@@ -427,9 +427,15 @@ constexpr int kComputeUnits = 256;
 constexpr int kPersistentFactor = 2;  // column groups per workgroup from which on workgroups walk
 
 
-void choose_shape(int m, int n, int* nt, int* depth) {
+void choose_shape(int m, int n, int k, int* nt, int* depth) {
   const int tiles = n / 16;
-  const float a_weight = (m > 4) ? 0.2f : 0.05f;  // cost of fetching the activations relative to one tile's work
+  // cost of fetching the activation rows relative to one tile's work: small while they are staged once per
+  // workgroup; when K is too long for that they are fetched again for every column group, 16 rows x 2 bytes
+  // against a tile's 16 columns x 1/2 byte per k
+  int rows = 1;
+  while (rows < m) rows *= 2;
+  const bool rows_fit = static_cast<size_t>(rows) * static_cast<size_t>(k) * 2 <= kMaxLdsBytes;
+  const float a_weight = !rows_fit ? static_cast<float>(rows) / 4.0f : (m > 4) ? 0.2f : 0.05f;
   float best = 0.f;
   *nt = 1;
   for (int t = 1; t <= 3; ++t) {
@@ -584,7 +590,7 @@ int launch_shape(const blkq4_gemm_args* a) {
   int status;
   if (launch_independent_waves<BS, HAS_ZP, ROW>(a, &status)) return status;
   int nt, depth;
-  choose_shape(a->m, a->n, &nt, &depth);
+  choose_shape(a->m, a->n, a->k, &nt, &depth);
   if (ROW) {
     // blocks along N: 28 registers of packed weights, scales and zero-points per slot and tile, so one tile
     return (depth == 8) ? launch_waves<BS, HAS_ZP, ROW, 8, 1>(a) : launch_waves<BS, HAS_ZP, ROW, 4, 1>(a);
