@@ -45,7 +45,7 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k) {
   {
     // its workgroups take 4, 2 or 1 column tiles of 16 (blocks along N: 1), as blkq4_skinny.hip chooses them
     const long tiles = static_cast<long>(n / 16) * row_groups;
-    const long per_group = !column_wise ? 1 : tiles >= 1024 ? 4 : tiles >= 512 ? 2 : 1;
+    const long per_group = !column_wise ? 1 : tiles >= 640 ? 4 : tiles >= 320 ? 2 : 1;
     const long streaming_groups = row_groups * ((n / 16 + per_group - 1) / per_group);
     if (streaming_groups > 256) {
       streaming_us *= static_cast<double>((streaming_groups + 255) / 256) / (static_cast<double>(streaming_groups) / 256.0);

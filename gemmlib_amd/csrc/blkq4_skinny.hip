@@ -580,11 +580,12 @@ template <int BS, bool HAS_ZP, bool ROW>
 int launch_shape(const blkq4_gemm_args* a) {
   if (a->m > 16) {
     // Every workgroup fetches the 32 rows of its group for all of K, so wide workgroups (more column tiles)
-    // mean less activation traffic; but there should be a workgroup for every compute unit.
+    // mean less activation traffic; but there should be a workgroup for most compute units (measured: four
+    // tiles per workgroup from 160 workgroups of four on, two from 160 of two on).
     const int row_groups = (a->m + 31) / 32;
     const long tiles = static_cast<long>(a->n / 16) * row_groups;
-    if (tiles >= 4 * kComputeUnits) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 4>(a, row_groups);
-    if (tiles >= 2 * kComputeUnits) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 2>(a, row_groups);
+    if (tiles >= 640) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 4>(a, row_groups);
+    if (tiles >= 320) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 2>(a, row_groups);
     return launch_rows<BS, HAS_ZP, ROW, 1>(a, row_groups);
   }
   int status;
