@@ -39,10 +39,11 @@ CONFIGS = {
     "C2r": (1, 4096, 4096, 64, False, "hbm"),
     "M128": (128, 4096, 4096, 64, True, "hbm"),
     "V128K": (1, 4096, 128256, 64, False, "hbm"),
+    "B16": (16, 8192, 28672, 64, True, "hbm"),
 }
 # workloads whose kernels run long enough for the clocks to matter: replayed untimed for a while before the
 # timed replay (a few milliseconds after an idle gap run at ramping clocks)
-SETTLE_SECONDS = {"V128K": 0.4}
+SETTLE_SECONDS = {"V128K": 0.4, "B16": 0.4}
 COLUMN_WISE = {"C4r": False, "C2r": False}
 DESCRIPTION = {
     "C1": "C1 CPU-runnable case M=64 K=1024 N=1024 bs32 asym",
@@ -54,6 +55,7 @@ DESCRIPTION = {
     "C2r": "C2 shape with blocks along N (column_wise_blocking=false) M=1 K=4096 N=4096 bs64 sym",
     "M128": "mid-size batch M=128 K=4096 N=4096 bs64 asym (streaming kernel in four row groups)",
     "V128K": "vocabulary projection GEMV M=1 K=4096 N=128256 bs64 sym (waves with a column tile of their own)",
+    "B16": "batch-16 decode on a wide layer M=16 K=8192 N=28672 bs64 asym (rows staged per slice)",
 }
 
 
@@ -347,7 +349,7 @@ def main(argv=None) -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r,C2r,M128,V128K")
+    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r,C2r,M128,V128K,B16")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-context", action="store_true", help="skip the floors and the library comparison")
     args = ap.parse_args(argv)
