@@ -590,6 +590,18 @@ int launch_shape(const blkq4_gemm_args* a) {
   }
   int status;
   if (launch_independent_waves<BS, HAS_ZP, ROW>(a, &status)) return status;
+  if constexpr (!ROW) {
+    // K too long for the rows to stay in LDS, wide N: the rows are staged per slice and fetched again for every
+    // column group, so a workgroup takes four column tiles; two slices in flight per wave keep the slots small
+    // enough for several workgroups per compute unit (M = 16, K = 8192: N = 14336 24.3 -> 17.6 us with eight
+    // waves, N = 28672 43.1 -> 34.1 us with four).
+    int rows_log2 = 0;
+    while ((1 << rows_log2) < a->m) ++rows_log2;
+    const bool rows_fit = ((static_cast<size_t>(a->k) * 2) << rows_log2) <= kMaxLdsBytes;
+    const int tiles = a->n / 16;
+    if (!rows_fit && tiles >= 1536) return launch_kernel<BS, HAS_ZP, ROW, 2, 4, 1, 4, kRowsPerSlotInLds>(a, rows_log2);
+    if (!rows_fit && tiles >= 832) return launch_kernel<BS, HAS_ZP, ROW, 2, 4, 1, 8, kRowsPerSlotInLds>(a, rows_log2);
+  }
   int nt, depth;
   choose_shape(a->m, a->n, a->k, &nt, &depth);
   if (ROW) {
