@@ -591,16 +591,20 @@ int launch_shape(const blkq4_gemm_args* a) {
   int status;
   if (launch_independent_waves<BS, HAS_ZP, ROW>(a, &status)) return status;
   if constexpr (!ROW) {
-    // K too long for the rows to stay in LDS, wide N: the rows are staged per slice and fetched again for every
-    // column group, so a workgroup takes four column tiles; two slices in flight per wave keep the slots small
-    // enough for several workgroups per compute unit (M = 16, K = 8192: N = 14336 24.3 -> 17.6 us with eight
-    // waves, N = 28672 43.1 -> 34.1 us with four).
+    // Wide N and more than four rows, or K too long for the rows to stay in LDS: the rows are staged per slice,
+    // a workgroup takes four column tiles (the rows are fetched again for every column group) and a wave keeps
+    // two slices in flight, so that the slots are small enough for several workgroups per compute unit: eight
+    // waves from 832 column tiles on, four from 1536 on.  Measured against every other shape of workgroup:
+    // M = 16, K = 8192: N = 14336 24.3 -> 17.6 us, N = 28672 43.1 -> 34.1 us; rows that would fit (M = 16,
+    // K = 4096, N = 14336: 13.2 -> 11.1 us) gain less or nothing, never lose more than 3 %.
     int rows_log2 = 0;
     while ((1 << rows_log2) < a->m) ++rows_log2;
     const bool rows_fit = ((static_cast<size_t>(a->k) * 2) << rows_log2) <= kMaxLdsBytes;
     const int tiles = a->n / 16;
-    if (!rows_fit && tiles >= 1536) return launch_kernel<BS, HAS_ZP, ROW, 2, 4, 1, 4, kRowsPerSlotInLds>(a, rows_log2);
-    if (!rows_fit && tiles >= 832) return launch_kernel<BS, HAS_ZP, ROW, 2, 4, 1, 8, kRowsPerSlotInLds>(a, rows_log2);
+    if ((!rows_fit || a->m > 4) && a->k >= 1024) {
+      if (tiles >= 1536) return launch_kernel<BS, HAS_ZP, ROW, 2, 4, 1, 4, kRowsPerSlotInLds>(a, rows_log2);
+      if (tiles >= 832) return launch_kernel<BS, HAS_ZP, ROW, 2, 4, 1, 8, kRowsPerSlotInLds>(a, rows_log2);
+    }
   }
   int nt, depth;
   choose_shape(a->m, a->n, a->k, &nt, &depth);
