@@ -526,6 +526,18 @@ int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
   }
 }
 
+// Slices that `waves` waves with rings of `depth` slices request for one column group: every wave asks for
+// whole rings, also when it has fewer slices left.
+int requested_slices(int k, int waves, int depth) {
+  const int slices = (k / 32 + 3) / 4;
+  int total = 0;
+  for (int w = 0; w < waves; ++w) {
+    const int mine = (slices - w + waves - 1) / waves;
+    total += (mine + depth - 1) / depth * depth;
+  }
+  return total;
+}
+
 // M <= 16, enough column tiles to give every wave the chip can hold one of its own, and rows small enough for
 // several workgroups per compute unit: the waves do not split K, each streams all of K for its own tile:
 // no sums across waves, no barriers, and a ring that stays full from the first slice to the last.
@@ -536,8 +548,12 @@ bool launch_independent_waves(const blkq4_gemm_args* a, int* status) {
   const size_t a_bytes = (((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023};
   // measured break-even against workgroups that split K and walk (blocks along N gain more: their sixteen-wave
   // kernel has no walking variant)
-  constexpr int kIndependentMinTiles = ROW ? 896 : 2000;
   constexpr size_t kIndependentMaxRowBytes = (ROW ? 32 : 16) * 1024;
+  // (from 832 tiles on when K is no multiple of what the splitting waves' rings hold, which then ask for a
+  // fifth more slices than there are: K = 5120, N = 13824: 14.5 -> 12.7 us)
+  const int slices = (a->k / 32 + 3) / 4;
+  const bool rings_fit_k = 5 * requested_slices(a->k, 16, 2) < 6 * slices || 5 * requested_slices(a->k, 8, 4) < 6 * slices;
+  const int kIndependentMinTiles = ROW ? 896 : rings_fit_k ? 2000 : 832;
   if (a->n / 16 < kIndependentMinTiles || a_bytes > kIndependentMaxRowBytes ||
       (reinterpret_cast<uintptr_t>(a->c) & 7u) != 0) {
     return false;
@@ -555,8 +571,16 @@ int launch_waves(const blkq4_gemm_args* a) {
   while ((1 << rows_log2) < a->m) ++rows_log2;
   const size_t a_bytes = (((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023};
   // sixteen waves when there is enough K: each wave has less to convert after its last load has arrived,
-  // and more of that work overlaps the loads of the other waves
+  // and more of that work overlaps the loads of the other waves.  With more workgroups than compute units,
+  // eight waves: smaller workgroups fill the units more evenly (M = 1, K = 4096, N = 14336: 11.4 -> 9.5 us),
+  // unless their rings would ask for many more slices than K has.
   if (a->k >= 4096 && a_bytes <= kMaxLdsBytes) {
+    constexpr int kD8 = DEPTH > 4 ? 4 : DEPTH;
+    const int col_groups = (a->n / 16 + NT - 1) / NT;
+    if (!ROW && col_groups > kComputeUnits &&
+        20 * requested_slices(a->k, 8, kD8) <= 21 * requested_slices(a->k, 16, 2)) {
+      return launch_kernel<BS, HAS_ZP, ROW, kD8, NT, 1, 8, kRowsWholeInLds>(a, rows_log2);
+    }
     return launch_kernel<BS, HAS_ZP, ROW, 2, NT, 1, 16, kRowsWholeInLds>(a, rows_log2);
   }
   if (a->k >= 1024) {

@@ -96,6 +96,7 @@ VERY_WIDE_CASES = [
     (64, False, 1, 32000, 4096), (32, True, 2, 32032, 4032), (16, True, 4, 32768, 320), (64, True, 1, 32000, 8192),
     (64, False, 1, 14336, 4096), (32, True, 2, 16416, 4160), (32, False, 16, 32032, 256), (16, True, 9, 32000, 448),
     (64, True, 8, 32800, 4096), (32, True, 16, 16416, 8256), (32, True, 96, 5440, 4160), (16, False, 12, 28672, 1088),
+    (64, False, 1, 13824, 5120), (32, True, 4, 14336, 4096), (16, True, 3, 22016, 4096), (32, True, 2, 13856, 5184),
 ]
 
 
