@@ -20,6 +20,8 @@ EXPORTED_SYMBOLS = (
     "blkq4_fp16_quant_sm80",
     "blkq4_fp16_quant_size_sm80",
     "blkq4_fp16_repack_sm80",
+    "blkq4_bf16_quant_sm80",
+    "blkq4_bf16_gemm_sm80",
     "blkq4_error_message_create",
     "blkq4_error_message_cstr",
     "blkq4_error_message_destroy",
@@ -59,6 +61,10 @@ def load() -> ctypes.CDLL:
     L.blkq4_fp16_quant_size_sm80.restype = i
     L.blkq4_fp16_repack_sm80.argtypes = [i, i, i, vp, vp, sz, vp, sz, vp]
     L.blkq4_fp16_repack_sm80.restype = i
+    L.blkq4_bf16_quant_sm80.argtypes = L.blkq4_fp16_quant_sm80.argtypes
+    L.blkq4_bf16_quant_sm80.restype = i
+    L.blkq4_bf16_gemm_sm80.argtypes = L.blkq4_fp16_gemm_bias_sm80.argtypes
+    L.blkq4_bf16_gemm_sm80.restype = i
     L.blkq4_error_message_create.restype = vp
     L.blkq4_error_message_cstr.argtypes = [vp]
     L.blkq4_error_message_cstr.restype = ctypes.c_char_p
@@ -128,26 +134,33 @@ def _stream_ptr(stream):
 
 
 def quant(block_size: int, column_wise: bool, weights_nk, q_weights, q_scales, q_zp=None, stream=None,
-          rows=None, columns=None, ld=None):
-    """``blkq4_fp16_quant_sm80`` on device tensors.  ``weights_nk`` is the torch ``[out, in]`` fp16
-    tensor (rows = in_features = ``weights_nk.shape[1]``)."""
+          rows=None, columns=None, ld=None, bf16=False):
+    """``blkq4_fp16_quant_sm80`` on device tensors (``bf16=True``: ``blkq4_bf16_quant_sm80``).  ``weights_nk``
+    is the torch ``[out, in]`` tensor (rows = in_features = ``weights_nk.shape[1]``)."""
     L = load()
     err = _ErrMsg(L)
     columns = weights_nk.shape[0] if columns is None else columns
     rows = weights_nk.shape[1] if rows is None else rows
     ld = weights_nk.stride(0) if ld is None else ld
-    rc = L.blkq4_fp16_quant_sm80(block_size, column_wise, rows, columns, ld, _stream_ptr(stream),
+    entry = L.blkq4_bf16_quant_sm80 if bf16 else L.blkq4_fp16_quant_sm80
+    rc = entry(block_size, column_wise, rows, columns, ld, _stream_ptr(stream),
                                  _ptr(weights_nk), _nbytes(weights_nk), _ptr(q_weights), _nbytes(q_weights),
                                  _ptr(q_scales), _nbytes(q_scales), _ptr(q_zp), _nbytes(q_zp), err.h)
     _check(rc, err)
 
 
 def gemm(block_size: int, column_wise: bool, m: int, n: int, k: int, a, q_weights, q_scales, q_zp, out,
-         stream=None, bias=None):
-    """``blkq4_fp16_gemm_sm80`` on device tensors; with ``bias`` (fp16 ``[n]``) ``blkq4_fp16_gemm_bias_sm80``."""
+         stream=None, bias=None, bf16=False):
+    """``blkq4_fp16_gemm_sm80`` on device tensors; with ``bias`` (fp16 ``[n]``) ``blkq4_fp16_gemm_bias_sm80``;
+    ``bf16=True``: ``blkq4_bf16_gemm_sm80`` (bias optional)."""
     L = load()
     err = _ErrMsg(L)
-    if bias is None:
+    if bf16:
+        rc = L.blkq4_bf16_gemm_sm80(block_size, column_wise, m, n, k, _stream_ptr(stream), _ptr(a), _nbytes(a),
+                                    _ptr(q_weights), _nbytes(q_weights), _ptr(q_scales), _nbytes(q_scales),
+                                    _ptr(q_zp), _nbytes(q_zp), _ptr(bias), _nbytes(bias), _ptr(out),
+                                    _nbytes(out), err.h)
+    elif bias is None:
         rc = L.blkq4_fp16_gemm_sm80(block_size, column_wise, m, n, k, _stream_ptr(stream), _ptr(a), _nbytes(a),
                                     _ptr(q_weights), _nbytes(q_weights), _ptr(q_scales), _nbytes(q_scales),
                                     _ptr(q_zp), _nbytes(q_zp), _ptr(out), _nbytes(out), err.h)

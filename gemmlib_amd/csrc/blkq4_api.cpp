@@ -115,15 +115,26 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_size_sm80(int block_size, bool colu
                     quant_meta_size, err);
 }
 
-// reference: src/blkq4_f16_gemm_sm80.cu:465-531 and :205-314 (blkq4_quant_sm80_T)
-extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_sm80(int block_size, bool column_wise_blocking, int rows,
-                                                  int columns, int leadingDimension, void* stream,
-                                                  void const* weights, size_t weights_size,
-                                                  void* quant_weights, size_t quant_weights_size,
-                                                  void* quant_scales, size_t quant_scales_size,
-                                                  void* offsets, size_t offsets_size,
-                                                  void* err_msg_ptr) {
+namespace {
+
+// bf16 has one blocking, the one the GEMV and GEMM configurations of the fp16 path are quoted on
+bool bf16_blocking_ok(bool bf16, bool column_wise_blocking, std::string* err) {
+  if (bf16 && !column_wise_blocking) {
+    set_error(err, "bf16 is implemented for column-wise blocking only");
+    return false;
+  }
+  return true;
+}
+
+// reference: src/blkq4_f16_gemm_sm80.cu:465-531 and :205-314 (blkq4_quant_sm80_T); bf16: the element type
+// the reference's template anticipates (src/mickey/blk_q4/f16_quant_sm80.cuh:16) and its entry points
+// reject (src/blkq4_f16_gemm_sm80.cu:53)
+int quant_entry(bool bf16, int block_size, bool column_wise_blocking, int rows, int columns, int leadingDimension,
+                void* stream, void const* weights, size_t weights_size, void* quant_weights,
+                size_t quant_weights_size, void* quant_scales, size_t quant_scales_size, void* offsets,
+                size_t offsets_size, void* err_msg_ptr) {
   auto* err = static_cast<std::string*>(err_msg_ptr);
+  if (!bf16_blocking_ok(bf16, column_wise_blocking, err)) return -1;
   if (!supported_block_size(block_size)) {
     set_error(err, "Unsupported block size: " + std::to_string(block_size));
     return -1;
@@ -185,15 +196,43 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_sm80(int block_size, bool column_wi
   args.scales = quant_scales;
   args.zero_points = has_offsets ? offsets : nullptr;
   args.stream = stream;
+  args.bf16 = bf16 ? 1 : 0;
   if (int code = blkq4_dev_prepack(&args)) return device_failure(code, err);
   return 0;
+}
+
+}  // namespace
+
+extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_sm80(int block_size, bool column_wise_blocking, int rows,
+                                                  int columns, int leadingDimension, void* stream,
+                                                  void const* weights, size_t weights_size,
+                                                  void* quant_weights, size_t quant_weights_size,
+                                                  void* quant_scales, size_t quant_scales_size,
+                                                  void* offsets, size_t offsets_size,
+                                                  void* err_msg_ptr) {
+  return quant_entry(false, block_size, column_wise_blocking, rows, columns, leadingDimension, stream, weights,
+                     weights_size, quant_weights, quant_weights_size, quant_scales, quant_scales_size, offsets,
+                     offsets_size, err_msg_ptr);
+}
+
+// the same quantizer for bf16 weights and scales; sizes as blkq4_fp16_quant_size_sm80 gives them
+extern "C" BLKQ4_EXPORT int blkq4_bf16_quant_sm80(int block_size, bool column_wise_blocking, int rows,
+                                                  int columns, int leadingDimension, void* stream,
+                                                  void const* weights, size_t weights_size,
+                                                  void* quant_weights, size_t quant_weights_size,
+                                                  void* quant_scales, size_t quant_scales_size,
+                                                  void* offsets, size_t offsets_size,
+                                                  void* err_msg_ptr) {
+  return quant_entry(true, block_size, column_wise_blocking, rows, columns, leadingDimension, stream, weights,
+                     weights_size, quant_weights, quant_weights_size, quant_scales, quant_scales_size, offsets,
+                     offsets_size, err_msg_ptr);
 }
 
 namespace {
 
 // reference: src/blkq4_f16_gemm_sm80.cu:319-429 and :38-153 (blkq4_gemm_sm80_T); bias_ptr == nullptr or
 // bias_size == 0: no bias
-int gemm_entry(int block_size, bool column_wise_blocking, int m, int n, int k, void* stream, void const* act_ptr,
+int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int n, int k, void* stream, void const* act_ptr,
                size_t a_size, void const* weights_ptr, size_t weights_size, void const* scales_ptr,
                size_t scales_size, void const* offsets_ptr, size_t offsets_size, void const* bias_ptr,
                size_t bias_size, void* output_ptr, size_t output_size, void* err_msg_ptr) {
@@ -203,6 +242,7 @@ int gemm_entry(int block_size, bool column_wise_blocking, int m, int n, int k, v
     return -1;
   }
   const bool has_offsets = offsets_ptr != nullptr && offsets_size > 0;
+  if (!bf16_blocking_ok(bf16, column_wise_blocking, err)) return -1;
 
   if (m <= 0 || n <= 0 || k <= 0) {
     set_error(err, "Empty problem size: " + std::to_string(m) + "x" + std::to_string(n) + "x" +
@@ -287,6 +327,17 @@ int gemm_entry(int block_size, bool column_wise_blocking, int m, int n, int k, v
   args.c = output_ptr;
   args.bias = has_bias ? bias_ptr : nullptr;
   args.stream = stream;
+  if (bf16) {
+    // bf16 has the weight-streaming kernel only, which takes up to 1024 rows at a time
+    constexpr int kChunk = 1024;
+    for (int m0 = 0; m0 < m; m0 += kChunk) {
+      args.m = (m - m0 < kChunk) ? m - m0 : kChunk;
+      args.a = static_cast<const char*>(act_ptr) + static_cast<size_t>(m0) * K * 2;
+      args.c = static_cast<char*>(output_ptr) + static_cast<size_t>(m0) * N * 2;
+      if (const int code = blkq4_dev_skinny_bf16(&args)) return device_failure(code, err);
+    }
+    return 0;
+  }
   // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
   const int code = streaming_kernel_takes(column_wise_blocking, m, n, k) ? blkq4_dev_skinny(&args) : blkq4_dev_gemm(&args);
   if (code) return device_failure(code, err);
@@ -302,7 +353,7 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_sm80(int block_size, bool column_wis
                                                  size_t scales_size, void const* offsets_ptr,
                                                  size_t offsets_size, void* output_ptr,
                                                  size_t output_size, void* err_msg_ptr) {
-  return gemm_entry(block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
+  return gemm_entry(false, block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
                     scales_ptr, scales_size, offsets_ptr, offsets_size, nullptr, 0, output_ptr, output_size,
                     err_msg_ptr);
 }
@@ -317,9 +368,23 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_bias_sm80(int block_size, bool colum
                                                       size_t offsets_size, void const* bias_ptr,
                                                       size_t bias_size, void* output_ptr,
                                                       size_t output_size, void* err_msg_ptr) {
-  return gemm_entry(block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
+  return gemm_entry(false, block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
                     scales_ptr, scales_size, offsets_ptr, offsets_size, bias_ptr, bias_size, output_ptr,
                     output_size, err_msg_ptr);
+}
+
+// bf16 activations, scales, bias and output (fp32 accumulation, one rounding of the output, then the bias the
+// way a tensor library adds two bf16 tensors); bias_ptr == nullptr or bias_size == 0: no bias
+extern "C" BLKQ4_EXPORT int blkq4_bf16_gemm_sm80(int block_size, bool column_wise_blocking, int m, int n, int k,
+                                                 void* stream, void const* act_ptr, size_t a_size,
+                                                 void const* weights_ptr, size_t weights_size,
+                                                 void const* scales_ptr, size_t scales_size,
+                                                 void const* offsets_ptr, size_t offsets_size,
+                                                 void const* bias_ptr, size_t bias_size, void* output_ptr,
+                                                 size_t output_size, void* err_msg_ptr) {
+  return gemm_entry(true, block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr,
+                    weights_size, scales_ptr, scales_size, offsets_ptr, offsets_size, bias_ptr, bias_size,
+                    output_ptr, output_size, err_msg_ptr);
 }
 
 extern "C" BLKQ4_EXPORT int blkq4_fp16_repack_sm80(int to_sm80, int rows, int columns, void* stream,

@@ -125,6 +125,46 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
   return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
 }
 
+// ---- bf16 (blocks along K only) ----------------------------------------------------------------------
+// Dequantized value: bf16( scale * (q - zp) ) with ONE rounding, the same definition as for fp16 with the
+// other 16-bit type.  A bf16 scale is m * 2^e with an 8-bit m, q and zp are below 16, so q * scale and
+// zp * scale are exact in fp32 and so is their difference (m * (q - zp) has at most 12 bits): one fma per
+// weight gives the exact product, the conversion to bf16 does the one rounding.  Per 8 weights: 1 shift,
+// 2 ands (nibbles to bytes), 8 byte -> float conversions, 8 fmas, 4 packed conversions to bf16.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));  // round to nearest even
+}
+
+struct Bf16Consts {
+  float scale;    // s
+  float neg_zps;  // -(zp * s), exact
+};
+__device__ __forceinline__ Bf16Consts make_bf16_consts(uint32_t scale_bits, uint32_t zp) {
+  Bf16Consts c;
+  c.scale = bf16_bits_to_float(scale_bits);
+  c.neg_zps = -(static_cast<float>(zp) * c.scale);
+  return c;
+}
+// One packed word (8 weights k0..k0+7 of one column) -> 8 bf16 in k order.  Nibble i of the word is weight
+// k0 + 2 i, nibble i + 4 weight k0 + 2 i + 1.
+__device__ __forceinline__ bf16x8_t dequant_word_bf16(uint32_t w, const Bf16Consts& c) {
+  const uint32_t lo = w & 0x0f0f0f0fu;         // nibbles 0, 2, 4, 6 as bytes
+  const uint32_t hi = (w >> 4) & 0x0f0f0f0fu;  // nibbles 1, 3, 5, 7
+  const uint32_t q[8] = {lo & 0xffu, (lo >> 16) & 0xffu, hi & 0xffu, (hi >> 16) & 0xffu,
+                         (lo >> 8) & 0xffu, lo >> 24, (hi >> 8) & 0xffu, hi >> 24};
+  bf16x8_t r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(q[i]), c.scale, c.neg_zps));
+  return r;
+}
+__device__ __forceinline__ bf16x8_t as_bf16x8(uint4 v) {
+  uint4_t t = {v.x, v.y, v.z, v.w};
+  return __builtin_bit_cast(bf16x8_t, t);
+}
+
 // c + bias the way an fp16 tensor library adds two fp16 tensors: in fp32, rounded to fp16 (the reference
 // module adds its bias to the fp16 output of the GEMM, python/ms_blkq4linear.py:26-27).
 __device__ __forceinline__ uint32_t add_bias_bits(uint32_t c, uint32_t bias) {
@@ -132,6 +172,21 @@ __device__ __forceinline__ uint32_t add_bias_bits(uint32_t c, uint32_t bias) {
 }
 __device__ __forceinline__ uint32_t add_bias_pair(uint32_t c, uint32_t bias) {
   return add_bias_bits(c & 0xffffu, bias & 0xffffu) | (add_bias_bits(c >> 16, bias >> 16) << 16);
+}
+
+// the same for either 16-bit type
+template <bool BF>
+__device__ __forceinline__ uint32_t float_to_bits(float f) {
+  return BF ? float_to_bf16_bits(f) : float_to_half_bits(f);
+}
+template <bool BF>
+__device__ __forceinline__ uint32_t add_bias_bits_t(uint32_t c, uint32_t bias) {
+  if (BF) return float_to_bf16_bits(bf16_bits_to_float(c) + bf16_bits_to_float(bias));
+  return add_bias_bits(c, bias);
+}
+template <bool BF>
+__device__ __forceinline__ uint32_t add_bias_pair_t(uint32_t c, uint32_t bias) {
+  return add_bias_bits_t<BF>(c & 0xffffu, bias & 0xffffu) | (add_bias_bits_t<BF>(c >> 16, bias >> 16) << 16);
 }
 
 }  // namespace blkq4

@@ -54,7 +54,18 @@ __device__ __forceinline__ float div_by_15(float x) {
 // nibble position of weight t (0..7) inside its 32-bit word
 __device__ __forceinline__ constexpr int nibble_shift(int t) { return 4 * ((t >> 1) + 4 * (t & 1)); }
 
-template <int BS, bool HAS_ZP, bool ALIGNED>
+// bf16: the other 16-bit type, the same arithmetic (a block's range is not bounded by 2^19 there, so the
+// division by 15 is the plain IEEE one)
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));  // round to nearest even
+}
+template <bool BF>
+__device__ __forceinline__ float bits_to_float(uint32_t b) { return BF ? bf16_bits_to_float(b) : half_bits_to_float(b); }
+template <bool BF>
+__device__ __forceinline__ uint16_t float_to_bits(float f) { return BF ? float_to_bf16_bits(f) : float_to_half_bits(f); }
+
+template <int BS, bool HAS_ZP, bool ALIGNED, bool BF = false>
 __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __restrict__ src, int K,
                                                            int N, int ld,
                                                            uint4* __restrict__ packed_w,
@@ -103,8 +114,8 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
     float v[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      v[2 * i] = half_bits_to_float(words[i] & 0xffffu);
-      v[2 * i + 1] = half_bits_to_float(words[i] >> 16);
+      v[2 * i] = bits_to_float<BF>(words[i] & 0xffffu);
+      v[2 * i + 1] = bits_to_float<BF>(words[i] >> 16);
     }
     // Range of the block: this lane's 8 weights, then the lanes that share the block.  The reference
     // scans in ascending k with strict compares, i.e. among equal values the first wins; that only
@@ -128,7 +139,7 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
       // reference: range2scalezp, f16_quant_sm80.cuh:96-122
       const float rmn = fminf(mn, 0.0f);
       const float rmx = fmaxf(mx, 0.0f);
-      const float scale_f = div_by_15(__fsub_rn(rmx, rmn));
+      const float scale_f = BF ? __fdiv_rn(__fsub_rn(rmx, rmn), 15.0f) : div_by_15(__fsub_rn(rmx, rmn));
       float zero_point_fp = rmn;
       if (scale_f != 0.0f) zero_point_fp = __fsub_rn(0.0f, __fdiv_rn(rmn, scale_f));
       if (zero_point_fp < 0.0f) {
@@ -138,11 +149,11 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
       } else {
         zp = round_0_to_15(zero_point_fp);
       }
-      scale_bits = float_to_half_bits(scale_f);
+      scale_bits = float_to_bits<BF>(scale_f);
     } else {
       // reference: range2scale, f16_quant_sm80.cuh:124-135
       const float m = fabsf(mx) > fabsf(mn) ? mx : mn;
-      scale_bits = float_to_half_bits(__fdiv_rn(m, -8.0f));
+      scale_bits = float_to_bits<BF>(__fdiv_rn(m, -8.0f));
       // (+-0) / -8 is a zero of the opposite sign (an all-zero block of +0 gives the scale -0.0): the
       // zero case takes its sign from the bits of the block's first weight, which is the value the
       // reference's scan ends with.
@@ -154,7 +165,7 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
     }
 
     // reference: f16_quant_sm80.cuh:291-297 (scale re-read after fp16 rounding; -0.0 counts as zero)
-    const float scale = half_bits_to_float(scale_bits);
+    const float scale = bits_to_float<BF>(scale_bits);
     const float reciprocal_scale = (scale != 0.0f) ? __fdiv_rn(1.0f, scale) : 0.0f;
     const float zp_f = static_cast<float>(zp);
     uint32_t word = 0;
@@ -440,7 +451,7 @@ int launch_prepack_rowwise(const blkq4_prepack_args* a) {
 
 template <int BS>
 int launch_prepack(const blkq4_prepack_args* a) {
-  if (!a->column_wise) return launch_prepack_rowwise<BS>(a);
+  if (!a->column_wise) return a->bf16 ? static_cast<int>(hipErrorInvalidValue) : launch_prepack_rowwise<BS>(a);
   const unsigned k_tiles = (a->rows + kTileK - 1) / kTileK;
   const dim3 grid(k_tiles * static_cast<unsigned>((a->columns + kTileN - 1) / kTileN));
   const dim3 block(kThreads);
@@ -451,6 +462,18 @@ int launch_prepack(const blkq4_prepack_args* a) {
   auto* zp = static_cast<uint8_t*>(a->zero_points);
   const bool aligned = (reinterpret_cast<uintptr_t>(a->src) & 15u) == 0 && (a->ld % 8) == 0;
   const bool has_zp = zp != nullptr;
+  if (a->bf16) {
+#define BLKQ4_LAUNCH(ZP_, AL_)                                                                                     \
+  hipLaunchKernelGGL((prepack_kernel<BS, ZP_, AL_, true>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, \
+                     pw, sc, zp, k_tiles)
+    if (has_zp) {
+      if (aligned) BLKQ4_LAUNCH(true, true); else BLKQ4_LAUNCH(true, false);
+    } else {
+      if (aligned) BLKQ4_LAUNCH(false, true); else BLKQ4_LAUNCH(false, false);
+    }
+#undef BLKQ4_LAUNCH
+    return static_cast<int>(hipGetLastError());
+  }
   if (has_zp) {
     if (aligned) {
       hipLaunchKernelGGL((prepack_kernel<BS, true, true>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, pw, sc, zp, k_tiles);

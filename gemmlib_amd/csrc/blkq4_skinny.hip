@@ -41,9 +41,23 @@
 #include "blkq4_device.h"
 #include "blkq4_gemm_common.h"
 
+// This file is compiled twice: as it is for fp16, and through blkq4_skinny_bf16.hip, which defines
+// BLKQ4_SKINNY_BF16 before including it, for bf16 activations, scales and outputs (blocks along K only).
+#ifdef BLKQ4_SKINNY_BF16
+#define BLKQ4_SKINNY_ENTRY blkq4_dev_skinny_bf16
+#else
+#define BLKQ4_SKINNY_ENTRY blkq4_dev_skinny
+#endif
+
 namespace {
 
 using namespace blkq4;
+
+#ifdef BLKQ4_SKINNY_BF16
+constexpr bool kBF = true;
+#else
+constexpr bool kBF = false;
+#endif
 
 // Where a wave finds its activation fragments.
 constexpr int kRowsWholeInLds = 1;   // all rows, all of K, staged once per workgroup
@@ -257,12 +271,12 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
           const int tile = (cgx * kTileWaves + wt) * NT + t;
           const int row = 16 * mt + nl;
           if (row < M && tile < tiles) {
-            uint32_t lo = float_to_half_bits(acc[t][mt][0]) | (static_cast<uint32_t>(float_to_half_bits(acc[t][mt][1])) << 16);
-            uint32_t hi = float_to_half_bits(acc[t][mt][2]) | (static_cast<uint32_t>(float_to_half_bits(acc[t][mt][3])) << 16);
+            uint32_t lo = float_to_bits<kBF>(acc[t][mt][0]) | (float_to_bits<kBF>(acc[t][mt][1]) << 16);
+            uint32_t hi = float_to_bits<kBF>(acc[t][mt][2]) | (float_to_bits<kBF>(acc[t][mt][3]) << 16);
             if (bias != nullptr) {
               const uint2 b = *reinterpret_cast<const uint2*>(bias + tile * 16 + 4 * g);
-              lo = add_bias_pair(lo, b.x);
-              hi = add_bias_pair(hi, b.y);
+              lo = add_bias_pair_t<kBF>(lo, b.x);
+              hi = add_bias_pair_t<kBF>(hi, b.y);
             }
             *reinterpret_cast<uint2*>(C + static_cast<size_t>(row) * N + tile * 16 + 4 * g) = make_uint2(lo, hi);
           }
@@ -290,8 +304,8 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       const int row = 16 * mt + (L & 15);
       if (row < M && cgx * NT + t < tiles) {
         const int col = cgx * (16 * NT) + 16 * t + 4 * (L >> 4) + e;
-        uint32_t h = float_to_half_bits(r);
-        if (bias != nullptr) h = add_bias_bits(h, bias[col]);
+        uint32_t h = float_to_bits<kBF>(r);
+        if (bias != nullptr) h = add_bias_bits_t<kBF>(h, bias[col]);
         C[static_cast<size_t>(row) * N + col] = static_cast<uint16_t>(h);
       }
     }
@@ -305,14 +319,14 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     const bool alt = rem != 0 && sl == last_slice;
     const uint32_t full = (slice < last_slice || (slice == last_slice && rem == 0)) ? 0xffffffffu : 0u;  // uniform
     const uint32_t okm = full | ((slice == last_slice) ? ok_last : 0u);
-      half8_t af[MT][4];
+      uint4 af[MT][4];  // eight 16-bit activations each
       if (A_LDS) {
         const uint8_t* ap = a_lds + (static_cast<uint32_t>(4 * sl) << (6 + rows_log2)) + (alt ? a_lane[1] : a_lane[0]);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            af[mt][j] = as_half8(*reinterpret_cast<const uint4*>(ap + mt * 1024 + ((j ^ a_swz) * 16)));
+            af[mt][j] = *reinterpret_cast<const uint4*>(ap + mt * 1024 + ((j ^ a_swz) * 16));
           }
       } else {
         // the rows of this slot were requested before its weights
@@ -323,12 +337,27 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            af[mt][j] = as_half8(*reinterpret_cast<const uint4*>(ap + mt * 1024 + ((j ^ a_swz) * 16)));
+            af[mt][j] = *reinterpret_cast<const uint4*>(ap + mt * 1024 + ((j ^ a_swz) * 16));
           }
       }
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         const uint32_t words[4] = {cur.w[t].x, cur.w[t].y, cur.w[t].z, cur.w[t].w};
+        if constexpr (kBF) {
+          // bf16: blocks along K only
+          Bf16Consts bc[kMeta];
+#pragma unroll
+          for (int q = 0; q < kMeta; ++q) bc[q] = make_bf16_consts(cur.sc[t][ROW ? 0 : q] & okm, cur.zp[t][ROW ? 0 : q]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const bf16x8_t wf = dequant_word_bf16(words[j], bc[(kMeta == 2) ? (j >> 1) : 0]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, as_bf16x8(af[mt][j]), acc[t][mt], 0, 0, 0);
+            }
+          }
+          continue;
+        }
         DequantConsts dc[kMeta];
         if (!ROW) {
 #pragma unroll
@@ -370,7 +399,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
           wf[4] = p[2][0]; wf[5] = p[2][1]; wf[6] = p[3][0]; wf[7] = p[3][1];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, af[mt][j], acc[t][mt], 0, 0, 0);
+            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, as_half8(af[mt][j]), acc[t][mt], 0, 0, 0);
           }
         }
       }
@@ -645,12 +674,17 @@ int launch_shape(const blkq4_gemm_args* a) {
 template <int BS>
 int launch_skinny(const blkq4_gemm_args* a) {
   if (a->column_wise) return a->zero_points ? launch_shape<BS, true, false>(a) : launch_shape<BS, false, false>(a);
-  return a->zero_points ? launch_shape<BS, true, true>(a) : launch_shape<BS, false, true>(a);
+  if constexpr (kBF) {
+    return static_cast<int>(hipErrorInvalidValue);
+  } else {
+    return a->zero_points ? launch_shape<BS, true, true>(a) : launch_shape<BS, false, true>(a);
+  }
 }
 
 }  // namespace
 
-extern "C" int blkq4_dev_skinny(const blkq4_gemm_args* a) {
+extern "C" int BLKQ4_SKINNY_ENTRY(const blkq4_gemm_args* a) {
+  if (kBF && !a->column_wise) return static_cast<int>(hipErrorInvalidValue);  // bf16: blocks along K only
   if (a->m < 1 || a->m > kStreamingMaxRows || (a->n % 16) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
   if (a->n > (1 << 26)) return static_cast<int>(hipErrorInvalidValue);  // a lane's offset inside a slice (up to 8 n rows of 16 bytes) is 32 bits wide
   if (!a->column_wise) {

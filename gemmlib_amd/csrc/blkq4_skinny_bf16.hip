@@ -1,0 +1,4 @@
+// The weight-streaming kernel for bf16 activations, scales and outputs: the same source as for fp16, with the
+// element type switched (conversion of the weights, MFMA instruction, rounding of the outputs, bias).
+#define BLKQ4_SKINNY_BF16 1
+#include "blkq4_skinny.hip"

@@ -128,6 +128,41 @@ int blkq4_fp16_repack_sm80(
     void* error_message);
 
 /**
+ * bf16: the quantizer and the GEMM above for bf16 weights, activations, scales, bias and output, the
+ * element type the reference's templates anticipate (reference: src/mickey/blk_q4/f16_quant_sm80.cuh:16,
+ * src/mickey/cutlass_ext/q4gemm/warp/quantb_mma_tensor_op.h:95-114) and its entry points reject
+ * (src/blkq4_f16_gemm_sm80.cu:53) -- so these two have no counterpart in the reference's C API.
+ * Same arguments, checks and messages as blkq4_fp16_quant_sm80 and blkq4_fp16_gemm_bias_sm80, every
+ * 16-bit buffer holding bf16; buffer sizes from blkq4_fp16_quant_size_sm80.  Arithmetic: the reference
+ * quantizer's with the scale rounded to bf16; weight = bf16(scale * (q - offset)) with one rounding; fp32
+ * accumulation, one rounding of the output to bf16, then the bias added in fp32 and rounded to bf16.
+ * Column-wise blocking only (column_wise_blocking = false fails with a message).  The packed weights
+ * and the offsets are interchangeable with the fp16 entry points'; the scales are not.
+ */
+int blkq4_bf16_quant_sm80(
+    int block_size,
+    bool column_wise_blocking,
+    int rows, int columns, int leadingDimension,
+    void* stream,
+    void const* weights, size_t weights_size,
+    void* quant_weights, size_t quant_weights_size,
+    void* quant_scales, size_t quant_scales_size,
+    void* offsets, size_t offsets_size,
+    void* error_message);
+int blkq4_bf16_gemm_sm80(
+  int block_size,
+  bool column_wise_blocking,
+  int m, int n, int k,
+  void* stream,
+  void const* act_ptr, size_t a_size,
+  void const* weights_ptr, size_t weights_size,
+  void const* scales_ptr, size_t scales_size,
+  void const* offsets_ptr, size_t offsets_size,
+  void const* bias_ptr, size_t bias_size,
+  void* output_ptr, size_t output_size,
+  void* error_message);
+
+/**
  * Helpers for callers that cannot construct a C++ std::string (ctypes, cgo, JNI ...): create an
  * error-message object to pass as `error_message`, read it, destroy it.  Host-only; no counterpart
  * in the reference, whose callers are all C++.

@@ -27,6 +27,13 @@
  *                            known-answer vectors held in tests/golden/.
  *   oracle_dequantize        pinned by test/blkq4_fp16_gemm_sm80_test.cu:309-328 (exact on the
  *                            known-answer data, so any mistake in indexing shows as a mismatch).
+ *   bf16 (`bf16 != 0` in the `_t` variants): the reference has no bf16 path and no vectors for one
+ *                            (src/blkq4_f16_gemm_sm80.cu:53 rejects the type), so these are the fp16
+ *                            functions with the 16-bit conversions exchanged.  The conversions are
+ *                            pinned exhaustively (all 65536 patterns up, round trip, and the rounding
+ *                            of every float between neighbouring bf16 values against numpy arithmetic);
+ *                            the quantizer by the same round-trip construction as fp16 on data exact
+ *                            in bf16; dequantize and GEMM against float64 numpy.
  *   oracle_gemm              textbook fp32-accumulate GEMM with one round-to-nearest fp16 conversion
  *                            (test/blkq4_fp16_gemm_sm80_test.cu:54-107,445-459); checked against a
  *                            float64 numpy matmul.
@@ -117,6 +124,29 @@ static inline uint16_t f2h(float f) {
 ORACLE_API float oracle_h2f(uint16_t h) { return h2f(h); }
 ORACLE_API uint16_t oracle_f2h(float f) { return f2h(f); }
 
+/* bfloat16 (the upper half of a binary32) <-> binary32, round-to-nearest-even.  The `_t` variants of the
+ * functions below take `bf16 != 0` to run the same algorithm on that 16-bit type instead of binary16. */
+static inline float b2f(uint16_t b) {
+  uint32_t bits = (uint32_t)b << 16;
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+static inline uint16_t f2b(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u); /* quiet NaN */
+  x += 0x7fffu + ((x >> 16) & 1u); /* ties to even; a carry out of the mantissa rounds up to the next exponent / inf */
+  return (uint16_t)(x >> 16);
+}
+
+ORACLE_API float oracle_b2f(uint16_t b) { return b2f(b); }
+ORACLE_API uint16_t oracle_f2b(float f) { return f2b(f); }
+
+static inline float e2f(uint16_t v, int bf16) { return bf16 ? b2f(v) : h2f(v); }
+static inline uint16_t f2e(float f, int bf16) { return bf16 ? f2b(f) : f2h(f); }
+
 /* ---------------------------------------------------------------------------------------------
  * Size query.  Reference: src/blkq4_f16_gemm_sm80.cu:155-203 (blkq4_quant_size_sm80_T) and
  * src/mickey/blk_q4/f16_quant_sm80.cuh:191-198.
@@ -147,7 +177,7 @@ ORACLE_API int oracle_quant_size(int block_size, int column_wise, int rows, int 
 
 /* :96-122 -- asymmetric: rectify the range to include 0, scale in fp32, zero-point from the
  * unrounded fp32 scale, roundf (half away from zero), then the scale is rounded to fp16. */
-static void range2scalezp(float mn, float mx, uint16_t* scale, uint8_t* zp) {
+static void range2scalezp(float mn, float mx, uint16_t* scale, uint8_t* zp, int bf16) {
   mn = fminf(mn, 0.0f);
   mx = fmaxf(mx, 0.0f);
   volatile float scale_f = (mx - mn) / 15.0f; /* volatile: forbid excess precision / reassociation */
@@ -163,13 +193,13 @@ static void range2scalezp(float mn, float mx, uint16_t* scale, uint8_t* zp) {
   } else {
     *zp = (uint8_t)roundf(zero_point_fp);
   }
-  *scale = f2h(scale_f);
+  *scale = f2e(scale_f, bf16);
 }
 
 /* :124-135 -- symmetric: the extreme value (ties go to min) divided by -8. */
-static void range2scale(float mn, float mx, uint16_t* scale) {
+static void range2scale(float mn, float mx, uint16_t* scale, int bf16) {
   float m = fabsf(mx) > fabsf(mn) ? mx : mn;
-  *scale = f2h(m / -8.0f);
+  *scale = f2e(m / -8.0f, bf16);
 }
 
 /* :286-313 -- one element. */
@@ -192,9 +222,9 @@ static inline uint8_t quantize_one(float v, float reciprocal_scale, uint8_t zp, 
  *   scales   fp16 column-major [K/kRow, N/kCol]: index meta_col*(K/kRow) + meta_row    (:277,290)
  *   zps      uint8, same indexing; NULL selects the symmetric quantizer (implicit zp 8, :292)
  */
-ORACLE_API int oracle_quantize(int block_size, int column_wise, int rows, int columns, int ld,
-                               const uint16_t* src, uint8_t* canon_w, uint16_t* canon_scales,
-                               uint8_t* canon_zps, int fused) {
+ORACLE_API int oracle_quantize_t(int block_size, int column_wise, int rows, int columns, int ld,
+                                 const uint16_t* src, uint8_t* canon_w, uint16_t* canon_scales,
+                                 uint8_t* canon_zps, int fused, int bf16) {
   int64_t wsz, msz;
   int err = oracle_quant_size(block_size, column_wise, rows, columns, &wsz, &msz);
   if (err) return err;
@@ -211,16 +241,16 @@ ORACLE_API int oracle_quantize(int block_size, int column_wise, int rows, int co
       float mx = -FLT_MAX;
       for (int i = mr * krow; i < (mr + 1) * krow; ++i) {
         for (int j = mc * kcol; j < (mc + 1) * kcol; ++j) {
-          const float v = h2f(src[(size_t)i + (size_t)j * ld]);
+          const float v = e2f(src[(size_t)i + (size_t)j * ld], bf16);
           if (v < mn) mn = v;
           if (v > mx) mx = v;
         }
       }
       const size_t meta_idx = (size_t)mc * meta_rows + mr;
       if (canon_zps == NULL) {
-        range2scale(mn, mx, &canon_scales[meta_idx]);
+        range2scale(mn, mx, &canon_scales[meta_idx], bf16);
       } else {
-        range2scalezp(mn, mx, &canon_scales[meta_idx], &canon_zps[meta_idx]);
+        range2scalezp(mn, mx, &canon_scales[meta_idx], &canon_zps[meta_idx], bf16);
       }
     }
   }
@@ -234,16 +264,22 @@ ORACLE_API int oracle_quantize(int block_size, int column_wise, int rows, int co
       for (int t = 0; t < 2; ++t) {
         const int meta_r = (i + t) / krow;
         const size_t meta_idx = (size_t)meta_c * meta_rows + meta_r;
-        const float scale = h2f(canon_scales[meta_idx]);
+        const float scale = e2f(canon_scales[meta_idx], bf16);
         const uint8_t zp = canon_zps ? canon_zps[meta_idx] : 8;
         volatile float reciprocal_scale = scale ? 1.0f / scale : 0.0f;
-        const float v = h2f(src[(size_t)(i + t) + (size_t)j * ld]);
+        const float v = e2f(src[(size_t)(i + t) + (size_t)j * ld], bf16);
         q[t] = quantize_one(v, reciprocal_scale, zp, fused);
       }
       canon_w[(size_t)j * (rows / 2) + i / 2] = (uint8_t)((q[0] & 0xf) | (q[1] << 4));
     }
   }
   return 0;
+}
+
+ORACLE_API int oracle_quantize(int block_size, int column_wise, int rows, int columns, int ld,
+                               const uint16_t* src, uint8_t* canon_w, uint16_t* canon_scales,
+                               uint8_t* canon_zps, int fused) {
+  return oracle_quantize_t(block_size, column_wise, rows, columns, ld, src, canon_w, canon_scales, canon_zps, fused, 0);
 }
 
 /* ---------------------------------------------------------------------------------------------
@@ -335,9 +371,9 @@ ORACLE_API int oracle_prepack_meta_sm80(int block_size, int column_wise, int row
  * (and test/blkq4_fp16_quant_sm80_test.cu:165-186): b = fp16( float(scale) * float(q - zp) ),
  * zp = 8 when there are no offsets.  Out: fp16 [K, N] column-major with leading dimension K.
  * ------------------------------------------------------------------------------------------- */
-ORACLE_API int oracle_dequantize(int block_size, int column_wise, int rows, int columns,
-                                 const uint8_t* canon_w, const uint16_t* canon_scales,
-                                 const uint8_t* canon_zps, uint16_t* b) {
+ORACLE_API int oracle_dequantize_t(int block_size, int column_wise, int rows, int columns,
+                                   const uint8_t* canon_w, const uint16_t* canon_scales,
+                                   const uint8_t* canon_zps, uint16_t* b, int bf16) {
   const int krow = column_wise ? block_size : 1;
   const int kcol = column_wise ? 1 : block_size;
   const int meta_rows = rows / krow;
@@ -348,11 +384,17 @@ ORACLE_API int oracle_dequantize(int block_size, int column_wise, int rows, int 
       const int offset = canon_zps ? canon_zps[meta_idx] : 8;
       const uint8_t byte = canon_w[(size_t)col * (rows / 2) + row / 2];
       const int w = ((row % 2 == 0) ? (byte & 0x0f) : (byte >> 4)) - offset;
-      const float scale = h2f(canon_scales[meta_idx]);
-      b[(size_t)col * rows + row] = f2h(scale * (float)w);
+      const float scale = e2f(canon_scales[meta_idx], bf16);
+      b[(size_t)col * rows + row] = f2e(scale * (float)w, bf16);
     }
   }
   return 0;
+}
+
+ORACLE_API int oracle_dequantize(int block_size, int column_wise, int rows, int columns,
+                                 const uint8_t* canon_w, const uint16_t* canon_scales,
+                                 const uint8_t* canon_zps, uint16_t* b) {
+  return oracle_dequantize_t(block_size, column_wise, rows, columns, canon_w, canon_scales, canon_zps, b, 0);
 }
 
 /* ---------------------------------------------------------------------------------------------
@@ -365,8 +407,8 @@ ORACLE_API int oracle_dequantize(int block_size, int column_wise, int rows, int 
  * additions within one output is ascending within each of 8 interleaved partial sums when
  * `strict_order` is 0 (fast, for the CPU baseline) and strictly ascending when it is 1.
  * ------------------------------------------------------------------------------------------- */
-ORACLE_API int oracle_gemm(int m, int n, int k, const uint16_t* a, const uint16_t* b, uint16_t* c,
-                           int strict_order) {
+ORACLE_API int oracle_gemm_t(int m, int n, int k, const uint16_t* a, const uint16_t* b, uint16_t* c,
+                             int strict_order, int bf16) {
   float* af = (float*)malloc((size_t)m * k * sizeof(float));
   float* bf = (float*)malloc((size_t)n * k * sizeof(float));
   if (!af || !bf) {
@@ -375,9 +417,9 @@ ORACLE_API int oracle_gemm(int m, int n, int k, const uint16_t* a, const uint16_
     return -1;
   }
 #pragma omp parallel for schedule(static)
-  for (int64_t i = 0; i < (int64_t)m * k; ++i) af[i] = h2f(a[i]);
+  for (int64_t i = 0; i < (int64_t)m * k; ++i) af[i] = e2f(a[i], bf16);
 #pragma omp parallel for schedule(static)
-  for (int64_t i = 0; i < (int64_t)n * k; ++i) bf[i] = h2f(b[i]);
+  for (int64_t i = 0; i < (int64_t)n * k; ++i) bf[i] = e2f(b[i], bf16);
 
 #pragma omp parallel for schedule(dynamic, 4) collapse(2)
   for (int j0 = 0; j0 < n; j0 += 8) {
@@ -401,13 +443,18 @@ ORACLE_API int oracle_gemm(int m, int n, int k, const uint16_t* a, const uint16_
           for (int t = 0; t < 16; ++t) acc += part[t];
           for (; kk < k; ++kk) acc += ar[kk] * bc[kk];
         }
-        c[(size_t)i * n + j] = f2h(acc);
+        c[(size_t)i * n + j] = f2e(acc, bf16);
       }
     }
   }
   free(af);
   free(bf);
   return 0;
+}
+
+ORACLE_API int oracle_gemm(int m, int n, int k, const uint16_t* a, const uint16_t* b, uint16_t* c,
+                           int strict_order) {
+  return oracle_gemm_t(m, n, k, a, b, c, strict_order, 0);
 }
 
 ORACLE_API int oracle_num_threads(void) {

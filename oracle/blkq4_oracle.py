@@ -41,10 +41,17 @@ def lib() -> ctypes.CDLL:
         vp, i, i64p = ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_int64)
         L.oracle_quant_size.argtypes = [i, i, i, i, i64p, i64p]
         L.oracle_quantize.argtypes = [i, i, i, i, i, vp, vp, vp, vp, i]
+        L.oracle_quantize_t.argtypes = [i, i, i, i, i, vp, vp, vp, vp, i, i]
         L.oracle_prepack_weights_sm80.argtypes = [i, i, vp, vp]
         L.oracle_prepack_meta_sm80.argtypes = [i, i, i, i, vp, vp, vp, vp]
         L.oracle_dequantize.argtypes = [i, i, i, i, vp, vp, vp, vp]
+        L.oracle_dequantize_t.argtypes = [i, i, i, i, vp, vp, vp, vp, i]
         L.oracle_gemm.argtypes = [i, i, i, vp, vp, vp, i]
+        L.oracle_gemm_t.argtypes = [i, i, i, vp, vp, vp, i, i]
+        L.oracle_b2f.argtypes = [ctypes.c_uint16]
+        L.oracle_b2f.restype = ctypes.c_float
+        L.oracle_f2b.argtypes = [ctypes.c_float]
+        L.oracle_f2b.restype = ctypes.c_uint16
         L.oracle_h2f.argtypes = [ctypes.c_uint16]
         L.oracle_h2f.restype = ctypes.c_float
         L.oracle_f2h.argtypes = [ctypes.c_float]
@@ -69,24 +76,44 @@ def quant_size(block_size, column_wise, rows, columns):
     return err, w.value, m.value
 
 
-def quantize(block_size, column_wise, weights_nk: np.ndarray, has_offsets: bool, fused: bool = True):
-    """Canonical quantized form of the torch-layout ``[N, K]`` fp16 weights.
+def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
+    """bf16 bit patterns (``uint16``) -> float32 (a bf16 is the upper half of a binary32)."""
+    return (bits.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bit patterns (``uint16``), round to nearest even, through the C oracle's scalar
+    conversion's vector form (the same integer rule, restated in numpy; NaNs are quieted)."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32)
+    r = ((u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    return np.where(nan, ((u >> np.uint32(16)) | np.uint32(0x40)).astype(np.uint16), r)
+
+
+def _elem_dtype(bf16: bool):
+    return np.uint16 if bf16 else np.float16
+
+
+def quantize(block_size, column_wise, weights_nk: np.ndarray, has_offsets: bool, fused: bool = True,
+             bf16: bool = False):
+    """Canonical quantized form of the torch-layout ``[N, K]`` fp16 weights (``bf16=True``: the weights
+    and the returned scales are bf16 bit patterns in ``uint16`` arrays).
 
     Reference: src/mickey/blk_q4/f16_quant_sm80.cuh:225-315.  Returns ``(canon_w, scales, zps)``:
     ``canon_w`` uint8 ``[N, K/2]`` (= col-major ``[K/2, N]``), ``scales`` fp16 ``[N/kCol, K/kRow]``
     (= col-major ``[K/kRow, N/kCol]``), ``zps`` uint8 of the same shape or ``None``.
     """
-    assert weights_nk.dtype == np.float16 and weights_nk.ndim == 2 and weights_nk.flags.c_contiguous
+    assert weights_nk.dtype == _elem_dtype(bf16) and weights_nk.ndim == 2 and weights_nk.flags.c_contiguous
     n, k = weights_nk.shape
     err, wsz, msz = quant_size(block_size, column_wise, k, n)
     if err:
         raise ValueError(f"oracle_quant_size failed: {err}")
     krow, kcol = (block_size, 1) if column_wise else (1, block_size)
     canon_w = np.empty((n, k // 2), np.uint8)
-    scales = np.empty((n // kcol, k // krow), np.float16)
+    scales = np.empty((n // kcol, k // krow), _elem_dtype(bf16))
     zps = np.empty((n // kcol, k // krow), np.uint8) if has_offsets else None
-    err = lib().oracle_quantize(block_size, int(column_wise), k, n, k, _p(weights_nk.view(np.uint16)),
-                                _p(canon_w), _p(scales.view(np.uint16)), _p(zps), int(fused))
+    err = lib().oracle_quantize_t(block_size, int(column_wise), k, n, k, _p(weights_nk.view(np.uint16)),
+                                  _p(canon_w), _p(scales.view(np.uint16)), _p(zps), int(fused), int(bf16))
     if err:
         raise ValueError(f"oracle_quantize failed: {err}")
     return canon_w, scales, zps
@@ -131,29 +158,34 @@ def quant_sm80(block_size, column_wise, weights_nk, has_offsets, fused=True):
     return prepack_weights_sm80(cw), ps, pz
 
 
-def dequantize(block_size, column_wise, canon_w, scales, zps) -> np.ndarray:
-    """Reference: test/blkq4_fp16_gemm_sm80_test.cu:309-328.  Returns fp16 ``[N, K]`` (= col-major ``[K, N]``)."""
+def dequantize(block_size, column_wise, canon_w, scales, zps, bf16: bool = False) -> np.ndarray:
+    """Reference: test/blkq4_fp16_gemm_sm80_test.cu:309-328.  Returns fp16 ``[N, K]`` (= col-major ``[K, N]``);
+    ``bf16=True``: scales in and weights out are bf16 bit patterns (``uint16``)."""
     n, k2 = canon_w.shape
-    b = np.empty((n, k2 * 2), np.float16)
-    lib().oracle_dequantize(block_size, int(column_wise), k2 * 2, n, _p(np.ascontiguousarray(canon_w)),
-                            _p(np.ascontiguousarray(scales).view(np.uint16)),
-                            _p(None if zps is None else np.ascontiguousarray(zps)), _p(b.view(np.uint16)))
+    assert scales.dtype == _elem_dtype(bf16)
+    b = np.empty((n, k2 * 2), _elem_dtype(bf16))
+    lib().oracle_dequantize_t(block_size, int(column_wise), k2 * 2, n, _p(np.ascontiguousarray(canon_w)),
+                              _p(np.ascontiguousarray(scales).view(np.uint16)),
+                              _p(None if zps is None else np.ascontiguousarray(zps)), _p(b.view(np.uint16)),
+                              int(bf16))
     return b
 
 
-def gemm(a_mk: np.ndarray, b_nk: np.ndarray, strict_order: bool = False) -> np.ndarray:
-    """fp16 ``C[M,N] = A[M,K] . B[K,N]`` with fp32 accumulation and one rounding to fp16.
+def gemm(a_mk: np.ndarray, b_nk: np.ndarray, strict_order: bool = False, bf16: bool = False) -> np.ndarray:
+    """fp16 ``C[M,N] = A[M,K] . B[K,N]`` with fp32 accumulation and one rounding to fp16 (``bf16=True``:
+    all three matrices are bf16 bit patterns in ``uint16`` arrays).
 
     Reference: test/blkq4_fp16_gemm_sm80_test.cu:54-107,445-459.  ``b_nk`` is the ``[N, K]`` array
     :func:`dequantize` returns.
     """
-    assert a_mk.dtype == np.float16 and b_nk.dtype == np.float16
+    assert a_mk.dtype == _elem_dtype(bf16) and b_nk.dtype == _elem_dtype(bf16)
     m, k = a_mk.shape
     n, k2 = b_nk.shape
     assert k == k2
-    c = np.empty((m, n), np.float16)
-    err = lib().oracle_gemm(m, n, k, _p(np.ascontiguousarray(a_mk).view(np.uint16)),
-                            _p(np.ascontiguousarray(b_nk).view(np.uint16)), _p(c.view(np.uint16)), int(strict_order))
+    c = np.empty((m, n), _elem_dtype(bf16))
+    err = lib().oracle_gemm_t(m, n, k, _p(np.ascontiguousarray(a_mk).view(np.uint16)),
+                              _p(np.ascontiguousarray(b_nk).view(np.uint16)), _p(c.view(np.uint16)),
+                              int(strict_order), int(bf16))
     if err:
         raise MemoryError("oracle_gemm")
     return c
