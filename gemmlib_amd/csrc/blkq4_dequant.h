@@ -127,10 +127,13 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
 
 // ---- bf16 (blocks along K only) ----------------------------------------------------------------------
 // Dequantized value: bf16( scale * (q - zp) ) with ONE rounding, the same definition as for fp16 with the
-// other 16-bit type.  A bf16 scale is m * 2^e with an 8-bit m, q and zp are below 16, so q * scale and
-// zp * scale are exact in fp32 and so is their difference (m * (q - zp) has at most 12 bits): one fma per
-// weight gives the exact product, the conversion to bf16 does the one rounding.  Per 8 weights: 1 shift,
-// 2 ands (nibbles to bytes), 8 byte -> float conversions, 8 fmas, 4 packed conversions to bf16.
+// other 16-bit type.  The nibbles become fp16 pairs (1024 + q) resp. (64 + q) exactly as above; each half is
+// then the fp16 operand of a mixed-precision fma with the scale and -(1024 + zp) * scale resp. -(64 + zp) * scale
+// in fp32 (v_fma_mix_f32 converts the fp16 operand exactly).  A bf16 scale is m * 2^e with an 8-bit m, 1024 + zp
+// has 11 bits, so the constant is exact in fp32 (19 bits) and the fma returns scale * (q - zp) exactly (12
+// bits); the packed conversion to bf16 does the one rounding.  Per 8 weights: 1 shift, 4 and-or, 8 fmas,
+// 4 packed conversions.  Scales beyond 2^118 overflow the constant (1039 * scale) although 15 * scale would
+// still be finite: such scales are outside the GEMM's range.
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
@@ -139,25 +142,33 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
 }
 
 struct Bf16Consts {
-  float scale;    // s
-  float neg_zps;  // -(zp * s), exact
+  float scale;   // s
+  float neg_c0;  // -(1024 + zp) * s, exact
+  float neg_c1;  // -(64 + zp) * s, exact
 };
 __device__ __forceinline__ Bf16Consts make_bf16_consts(uint32_t scale_bits, uint32_t zp) {
   Bf16Consts c;
   c.scale = bf16_bits_to_float(scale_bits);
-  c.neg_zps = -(static_cast<float>(zp) * c.scale);
+  c.neg_c0 = -(static_cast<float>(1024u + zp) * c.scale);
+  c.neg_c1 = -(static_cast<float>(64u + zp) * c.scale);
   return c;
 }
-// One packed word (8 weights k0..k0+7 of one column) -> 8 bf16 in k order.  Nibble i of the word is weight
-// k0 + 2 i, nibble i + 4 weight k0 + 2 i + 1.
-__device__ __forceinline__ bf16x8_t dequant_word_bf16(uint32_t w, const Bf16Consts& c) {
-  const uint32_t lo = w & 0x0f0f0f0fu;         // nibbles 0, 2, 4, 6 as bytes
-  const uint32_t hi = (w >> 4) & 0x0f0f0f0fu;  // nibbles 1, 3, 5, 7
-  const uint32_t q[8] = {lo & 0xffu, (lo >> 16) & 0xffu, hi & 0xffu, (hi >> 16) & 0xffu,
-                         (lo >> 8) & 0xffu, lo >> 24, (hi >> 8) & 0xffu, hi >> 24};
+// One packed word (8 weights k0..k0+7 of one column) -> 8 bf16 in k order.
+__device__ __forceinline__ bf16x8_t dequant_word_bf16(uint32_t w, const Bf16Consts& c, const DequantMasks& m) {
+  const uint32_t y = w >> 8;
+  const half2_t p0 = as_half2((w & m.lo_mask) | m.magic_1024);  // 1024 + q of k0, k0+1
+  const half2_t p1 = as_half2((w & m.hi_mask) | m.magic_64);    //   64 + q of k0+2, k0+3
+  const half2_t p2 = as_half2((y & m.lo_mask) | m.magic_1024);  // k0+4, k0+5
+  const half2_t p3 = as_half2((y & m.hi_mask) | m.magic_64);    // k0+6, k0+7
   bf16x8_t r;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) r[i] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(q[i]), c.scale, c.neg_zps));
+  r[0] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p0[0]), c.scale, c.neg_c0));
+  r[1] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p0[1]), c.scale, c.neg_c0));
+  r[2] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p1[0]), c.scale, c.neg_c1));
+  r[3] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p1[1]), c.scale, c.neg_c1));
+  r[4] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p2[0]), c.scale, c.neg_c0));
+  r[5] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p2[1]), c.scale, c.neg_c0));
+  r[6] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p3[0]), c.scale, c.neg_c1));
+  r[7] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p3[1]), c.scale, c.neg_c1));
   return r;
 }
 __device__ __forceinline__ bf16x8_t as_bf16x8(uint4 v) {

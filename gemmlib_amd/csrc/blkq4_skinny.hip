@@ -350,7 +350,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
           for (int q = 0; q < kMeta; ++q) bc[q] = make_bf16_consts(cur.sc[t][ROW ? 0 : q] & okm, cur.zp[t][ROW ? 0 : q]);
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const bf16x8_t wf = dequant_word_bf16(words[j], bc[(kMeta == 2) ? (j >> 1) : 0]);
+            const bf16x8_t wf = dequant_word_bf16(words[j], bc[(kMeta == 2) ? (j >> 1) : 0], masks);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
               acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, as_bf16x8(af[mt][j]), acc[t][mt], 0, 0, 0);
