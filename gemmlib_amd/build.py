@@ -27,7 +27,7 @@ PROBE_PATH = os.path.join(LIB_DIR, "libblkq4_probe.so")  # measurement aids for 
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-HIP_SOURCES = ["blkq4_prepack.hip", "blkq4_skinny.hip", "blkq4_skinny_bf16.hip", "blkq4_gemm.hip"]
+HIP_SOURCES = ["blkq4_prepack.hip", "blkq4_skinny.hip", "blkq4_skinny_bf16.hip", "blkq4_gemm.hip", "blkq4_gemm_bf16.hip"]
 HOST_SOURCES = ["blkq4_api.cpp"]
 
 # -ffp-contract=off: every fused multiply-add the quantizer needs is written as an explicit fmaf.

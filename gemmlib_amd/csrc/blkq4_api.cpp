@@ -327,19 +327,10 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
   args.c = output_ptr;
   args.bias = has_bias ? bias_ptr : nullptr;
   args.stream = stream;
-  if (bf16) {
-    // bf16 has the weight-streaming kernel only, which takes up to 1024 rows at a time
-    constexpr int kChunk = 1024;
-    for (int m0 = 0; m0 < m; m0 += kChunk) {
-      args.m = (m - m0 < kChunk) ? m - m0 : kChunk;
-      args.a = static_cast<const char*>(act_ptr) + static_cast<size_t>(m0) * K * 2;
-      args.c = static_cast<char*>(output_ptr) + static_cast<size_t>(m0) * N * 2;
-      if (const int code = blkq4_dev_skinny_bf16(&args)) return device_failure(code, err);
-    }
-    return 0;
-  }
   // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
-  const int code = streaming_kernel_takes(column_wise_blocking, m, n, k) ? blkq4_dev_skinny(&args) : blkq4_dev_gemm(&args);
+  const bool streaming = streaming_kernel_takes(column_wise_blocking, m, n, k);
+  const int code = bf16 ? (streaming ? blkq4_dev_skinny_bf16(&args) : blkq4_dev_gemm_bf16(&args))
+                        : (streaming ? blkq4_dev_skinny(&args) : blkq4_dev_gemm(&args));
   if (code) return device_failure(code, err);
   return 0;
 }

@@ -50,9 +50,24 @@
 #include "blkq4_device.h"
 #include "blkq4_gemm_common.h"
 
+// This file is compiled twice: as it is for fp16, and through blkq4_gemm_bf16.hip, which defines BLKQ4_GEMM_BF16
+// before including it, for bf16 activations, scales and outputs (blocks along K only).
+#ifdef BLKQ4_GEMM_BF16
+#define BLKQ4_GEMM_ENTRY blkq4_dev_gemm_bf16
+#else
+#define BLKQ4_GEMM_ENTRY blkq4_dev_gemm
+#endif
+
 namespace {
 
 using namespace blkq4;
+
+#ifdef BLKQ4_GEMM_BF16
+constexpr bool kBF = true;
+#else
+constexpr bool kBF = false;
+#endif
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kBK = 64;
 
@@ -325,7 +340,11 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   if (!ROW) {                                                                                       \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                                \
       _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                           \
-        (dc_)[t][q] = make_dequant_consts((dc_##_sc)[t][q], (dc_##_zp)[t][q]);                      \
+        if constexpr (kBF) {                                                                        \
+          (b##dc_)[t][q] = make_bf16_consts((dc_##_sc)[t][q], (dc_##_zp)[t][q]);                    \
+        } else {                                                                                    \
+          (dc_)[t][q] = make_dequant_consts((dc_##_sc)[t][q], (dc_##_zp)[t][q]);                    \
+        }                                                                                           \
       }                                                                                             \
     }                                                                                               \
   }
@@ -350,14 +369,33 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   // Blocks along N: word w_ of a lane's unit is rows 8 hh .. 8 hh + 7 (hh = w_ & 1) of 16-row group w_ / 2 of
   // the lane's 32 rows; pair p has its zero-points in byte pair hh of zero-point word p and its scales in
   // word 2 p + hh of the group (see blkq4_device.h for the packed order).
+  // bf16: PA is the two mixed-precision fmas of the pair (fp16 operand 1024 + q resp. 64 + q, fp32 scale and constant),
+  // PM the packed conversion of their results to bf16.
 #define BLKQ4_PIECE_PA(dc_, q_, w_, y_)                                                                       \
-  pt[y_] = pt[y_] + (ROW ? row_neg_c<HAS_ZP>(vec_word(mrow_z[(w_) >> 1][(y_) / 4], (y_) % 4), (y_) % 4, (w_)&1, rmasks) \
-                     : ((((y_) & 1) == 0) ? (dc_)[(y_) / 4][q_].neg_c0 : (dc_)[(y_) / 4][q_].neg_c1))
+  {                                                                                                           \
+    if constexpr (kBF) {                                                                                      \
+      const Bf16Consts& bc_ = (b##dc_)[(y_) / 4][q_];                                                         \
+      pf[y_][0] = __builtin_fmaf(static_cast<float>(pt[y_][0]), bc_.scale, (((y_) & 1) == 0) ? bc_.neg_c0 : bc_.neg_c1); \
+      pf[y_][1] = __builtin_fmaf(static_cast<float>(pt[y_][1]), bc_.scale, (((y_) & 1) == 0) ? bc_.neg_c0 : bc_.neg_c1); \
+    } else {                                                                                                  \
+      pt[y_] = pt[y_] + (ROW ? row_neg_c<HAS_ZP>(vec_word(mrow_z[(w_) >> 1][(y_) / 4], (y_) % 4), (y_) % 4, (w_)&1, rmasks) \
+                         : ((((y_) & 1) == 0) ? (dc_)[(y_) / 4][q_].neg_c0 : (dc_)[(y_) / 4][q_].neg_c1));   \
+    }                                                                                                         \
+  }
 #define BLKQ4_PIECE_PM(dst_, dc_, q_, w_, y_)                                                                \
-  wp[dst_][(y_) / 4][(y_) % 4] =                                                                             \
-      pt[y_] * (ROW ? as_half2(vec_word(mrow_s[(w_) >> 1][(y_) / 4][(2 * ((y_) % 4) + ((w_)&1)) >> 2],       \
-                                        (2 * ((y_) % 4) + ((w_)&1)) & 3))                                    \
-                    : (dc_)[(y_) / 4][q_].scale2)
+  {                                                                                                          \
+    if constexpr (kBF) {                                                                                     \
+      bf16x2_t v_;                                                                                           \
+      v_[0] = static_cast<__bf16>(pf[y_][0]);                                                                \
+      v_[1] = static_cast<__bf16>(pf[y_][1]);                                                                \
+      wp[dst_][(y_) / 4][(y_) % 4] = __builtin_bit_cast(half2_t, v_);                                        \
+    } else {                                                                                                 \
+      wp[dst_][(y_) / 4][(y_) % 4] =                                                                         \
+          pt[y_] * (ROW ? as_half2(vec_word(mrow_s[(w_) >> 1][(y_) / 4][(2 * ((y_) % 4) + ((w_)&1)) >> 2],   \
+                                            (2 * ((y_) % 4) + ((w_)&1)) & 3))                                \
+                        : (dc_)[(y_) / 4][q_].scale2);                                                       \
+    }                                                                                                        \
+  }
 #define BLKQ4_PIECE(dst_, words_, w_, dc_, q_, y_) \
   BLKQ4_PIECE_AO(words_, w_, y_);                  \
   BLKQ4_PIECE_PA(dc_, q_, w_, y_);                 \
@@ -372,9 +410,11 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   half8_t af[2][RT];      // activation fragments, double buffered over the k steps
   half2_t wp[2][NT][4];   // weight fragments (4 fp16 pairs each), double buffered
   half2_t pt[4 * NT];     // pieces of a fragment on their way through the conversion
+  float pf[4 * NT][2];    // bf16: the pieces as fp32 pairs between the fmas and the packed conversion
   uint32_t words[NT][4], nwords[NT][4];
   uint32_t dc_sc[NT][kMeta], dc_zp[NT][kMeta], ndc_sc[NT][kMeta], ndc_zp[NT][kMeta];
   DequantConsts dc[NT][kMeta], ndc[NT][kMeta];
+  Bf16Consts bdc[NT][kMeta], bndc[NT][kMeta];  // bf16: these instead
   uint4 mrow_s[2][NT][2], mrow_z[2][NT];  // blocks along N: meta of 16-row groups 2h (steps 0, 1) and 2h + 1 (steps 2, 3)
 
   {
@@ -401,7 +441,12 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
     _Pragma("unroll") for (int r = 0; r < RT; ++r) {                                               \
       _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                             \
         const int x_ = r * NT + t;                                                                 \
-        acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[t], af[cur_][r], acc[r][t], 0, 0, 0); \
+        if constexpr (kBF) {                                                                       \
+          acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wf_[t]),  \
+              __builtin_bit_cast(bf16x8_t, af[cur_][r]), acc[r][t], 0, 0, 0);                        \
+        } else {                                                                                   \
+          acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[t], af[cur_][r], acc[r][t], 0, 0, 0); \
+        }                                                                                          \
         if (t == NT - 1) BLKQ4_READ_A1(af[1 - (cur_)], nstage_, nj_, r);                           \
         _Pragma("unroll") for (int g2 = 0; g2 < 2 * NT; ++g2) {                                    \
           /* stage u of the pair's conversion is issued behind MFMA stage_slot(g2, u, ...) */      \
@@ -462,7 +507,10 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
 #pragma unroll
       for (int j = 0; j < 4; ++j) words[t][j] = nwords[t][j];
 #pragma unroll
-      for (int q = 0; q < kMeta; ++q) dc[t][q] = ndc[t][q];
+      for (int q = 0; q < kMeta; ++q) {
+        if constexpr (kBF) bdc[t][q] = bndc[t][q];
+        else dc[t][q] = ndc[t][q];
+      }
     }
   }
   if (PW == 0) wait_vmcnt<0>();  // the clamped re-fetches of the last tile are still in flight
@@ -504,10 +552,8 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
         for (int t = 0; t < NT; ++t) {
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            const uint32_t lo = float_to_half_bits(acc[r][t][4 * g + 0]) |
-                                (static_cast<uint32_t>(float_to_half_bits(acc[r][t][4 * g + 1])) << 16);
-            const uint32_t hi = float_to_half_bits(acc[r][t][4 * g + 2]) |
-                                (static_cast<uint32_t>(float_to_half_bits(acc[r][t][4 * g + 3])) << 16);
+            const uint32_t lo = float_to_bits<kBF>(acc[r][t][4 * g + 0]) | (float_to_bits<kBF>(acc[r][t][4 * g + 1]) << 16);
+            const uint32_t hi = float_to_bits<kBF>(acc[r][t][4 * g + 2]) | (float_to_bits<kBF>(acc[r][t][4 * g + 3]) << 16);
             lds_write_8(region + ((r - r0) * 32 + i) * kRowBytes + h * 8, t * 64 + g * 16, lo, hi);
           }
         }
@@ -517,8 +563,8 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
         const int row = it * kRowsPerStore + srow;  // inside the pass
         uint4 v = lds_read_16(region + srow * kRowBytes + chunk * 16, it * kRowsPerStore * kRowBytes);
         if (bias != nullptr) {
-          v = make_uint4(add_bias_pair(v.x, bias8.x), add_bias_pair(v.y, bias8.y), add_bias_pair(v.z, bias8.z),
-                         add_bias_pair(v.w, bias8.w));
+          v = make_uint4(add_bias_pair_t<kBF>(v.x, bias8.x), add_bias_pair_t<kBF>(v.y, bias8.y),
+                         add_bias_pair_t<kBF>(v.z, bias8.z), add_bias_pair_t<kBF>(v.w, bias8.w));
         }
         const int m = m0 + wm * (32 * RT) + r0 * 32 + row;
         if (m < M && col < N) *reinterpret_cast<uint4*>(C + static_cast<size_t>(m) * N + col) = v;
@@ -554,7 +600,9 @@ int launch_rt(const blkq4_gemm_args* a) {
   const long tiles = static_cast<long>((a->m + 255) / 256) * ((a->n + 255) / 256);
   const long small_tiles = static_cast<long>((a->m + 127) / 128) * ((a->n + 127) / 128);
   const long smallest_tiles = static_cast<long>((a->m + 63) / 64) * ((a->n + 127) / 128);
-  if (!a->column_wise) {
+  if constexpr (kBF) {
+    if (!a->column_wise) return static_cast<int>(hipErrorInvalidValue);  // bf16: blocks along K only
+  } else if (!a->column_wise) {
     // blocks along N (the streaming kernel takes the small row counts)
     if (tiles >= kComputeUnits) return launch_one<BS, HAS_ZP, 8, 2, 1, 4, 0, true>(a);
     if (smallest_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 2, 1, 1, 4, 4, true>(a);
@@ -586,7 +634,7 @@ int launch_bs(const blkq4_gemm_args* a) {
 
 }  // namespace
 
-extern "C" int blkq4_dev_gemm(const blkq4_gemm_args* a) {
+extern "C" int BLKQ4_GEMM_ENTRY(const blkq4_gemm_args* a) {
   if (a->m < 1 || (a->n % 32) != 0 || a->n < 32 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
   if (!a->column_wise && ((a->n % a->block_size) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 3u) != 0 ||
                           (reinterpret_cast<uintptr_t>(a->zero_points) & 3u) != 0)) {

@@ -1,0 +1,4 @@
+// The MFMA tile kernel for bf16 activations, scales and outputs: the same source as for fp16, with the element
+// type switched (conversion of the weights, MFMA instruction, rounding of the outputs, bias).
+#define BLKQ4_GEMM_BF16 1
+#include "blkq4_gemm.hip"

@@ -127,7 +127,8 @@ def test_quantizer_on_strided_and_unaligned_source(oracle, capi, device):
 
 # (block_size, has_offsets, m, n, k): the reference's column-wise cases (test/blkq4_fp16_gemm_sm80_test.cu:501-518),
 # then M = 1 and ragged M, wide N (waves with column tiles of their own, several column groups per workgroup),
-# long K (rows staged per slice), row groups of 32, and more than 1024 rows (the entry point walks over them)
+# long K (rows staged per slice), row groups of 32, and the tile kernel's shapes (256 x 256, 128 x 256, 128 x 128 and
+# 64 x 128 tiles, 32- and 64-row tiles on very wide layers, ragged edges)
 EXACT_CASES = [
     (16, False, 256, 672, 576), (16, True, 256, 672, 576), (64, False, 256, 1024, 576), (64, True, 256, 1024, 576),
     (16, False, 16, 672, 576), (16, True, 16, 672, 576), (64, False, 16, 1024, 576), (64, True, 16, 1024, 576),
@@ -135,7 +136,10 @@ EXACT_CASES = [
     (64, True, 33, 288, 320), (32, False, 100, 800, 448), (32, True, 300, 256, 64), (64, True, 1, 32000, 1024),
     (32, True, 2, 14336, 1024), (16, True, 9, 16416, 448), (32, True, 16, 64, 8192 + 64), (64, False, 9, 64, 12288),
     (32, True, 16, 11008, 1024), (64, True, 64, 4128, 320), (16, False, 96, 5440, 192), (32, True, 1500, 544, 128),
-    (64, False, 2048 + 5, 96, 192),
+    (64, False, 2048 + 5, 96, 192), (64, True, 4096, 4096, 128), (16, True, 4000, 4128, 64), (32, False, 4096, 4096, 192),
+    (64, True, 300, 4128, 192), (16, True, 500, 2080, 128), (32, False, 257, 4096, 64), (32, True, 1100, 4160, 128),
+    (64, True, 48, 28672, 256), (32, False, 64, 36864, 128), (16, False, 32, 28672, 2624), (32, True, 24, 36864, 2624),
+    (64, True, 768, 1056, 576), (16, True, 129, 1056, 576),
 ]
 
 
@@ -161,6 +165,7 @@ def test_gemm_exact_on_known_answer_construction(oracle, capi, device, bs, has_o
 @pytest.mark.parametrize("bs,has_offsets,m,n,k,seed", [
     (32, True, 64, 1024, 1024, 2235), (64, False, 1, 4096, 4096, 2236), (32, True, 16, 11008, 4096, 2237),
     (64, True, 128, 4096, 4096, 2238), (16, True, 8, 2048, 8192, 2239), (64, True, 1100, 1056, 512, 2240),
+    (64, True, 2048, 4096, 4096, 2241), (16, True, 512, 4096, 2048, 2242),
 ])
 def test_gemm_on_gaussian_data(oracle, capi, device, bs, has_offsets, m, n, k, seed):
     a, w = gaussian_bits(oracle, seed, m, n, k)
@@ -180,7 +185,8 @@ def test_gemm_on_gaussian_data(oracle, capi, device, bs, has_offsets, m, n, k, s
 
 @pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, False, 1, 4096, 512), (32, True, 16, 1056, 576),
                                                   (16, True, 64, 352, 256), (64, True, 2, 32000, 256),
-                                                  (32, True, 1100, 544, 128)])
+                                                  (32, True, 1100, 544, 128), (64, True, 300, 4128, 192),
+                                                  (16, True, 4096, 4096, 64)])
 def test_bias_equals_a_separate_add(oracle, capi, device, bs, has_offsets, m, n, k):
     """the bias is added to the bf16 output the way the tensor library adds two bf16 tensors (in fp32, one
     rounding), which is what the reference module does with fp16 (python/ms_blkq4linear.py:26-27)"""
