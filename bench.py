@@ -40,7 +40,10 @@ CONFIGS = {
     "M128": (128, 4096, 4096, 64, True, "hbm"),
     "V128K": (1, 4096, 128256, 64, False, "hbm"),
     "B16": (16, 8192, 28672, 64, True, "hbm"),
+    "C4b": (2048, 4096, 4096, 64, True, "mfma"),
+    "C2b": (1, 4096, 4096, 64, False, "hbm"),
 }
+BF16 = {"C4b", "C2b"}  # through blkq4_bf16_quant_sm80 / blkq4_bf16_gemm_sm80
 # workloads whose kernels run long enough for the clocks to matter: replayed untimed for a while before the
 # timed replay (a few milliseconds after an idle gap run at ramping clocks)
 SETTLE_SECONDS = {"V128K": 0.4, "B16": 0.4}
@@ -56,6 +59,8 @@ DESCRIPTION = {
     "M128": "mid-size batch M=128 K=4096 N=4096 bs64 asym (streaming kernel in four row groups)",
     "V128K": "vocabulary projection GEMV M=1 K=4096 N=128256 bs64 sym (waves with a column tile of their own)",
     "B16": "batch-16 decode on a wide layer M=16 K=8192 N=28672 bs64 asym (rows staged per slice)",
+    "C4b": "C4 shape in bf16 (blkq4_bf16_gemm_sm80) M=2048 K=4096 N=4096 bs64 asym",
+    "C2b": "C2 shape in bf16 (blkq4_bf16_gemm_sm80) M=1 K=4096 N=4096 bs64 sym",
 }
 
 
@@ -147,22 +152,24 @@ def timed_region(torch, launches, steps, warmup, settle_seconds=0.0):
 def make_problem(torch, capi, name, device, copies):
     m, k, n, bs, has_offsets, _ = CONFIGS[name]
     col = COLUMN_WISE.get(name, True)
+    bf = name in BF16
+    dtype = torch.bfloat16 if bf else torch.float16
     g = torch.Generator(device="cpu").manual_seed(1234 + list(CONFIGS).index(name))
-    a = torch.randn(m, k, generator=g, dtype=torch.float32).to(torch.float16).to(device)
+    a = torch.randn(m, k, generator=g, dtype=torch.float32).to(dtype).to(device)
     w_elems, meta_elems = capi.quant_size(bs, col, k, n)
     sets = []
     w_host = None
     for c in range(copies):
-        w_host = (torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).to(torch.float16)
+        w_host = (torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).to(dtype)
         w = w_host.to(device)
         q_w = torch.empty(w_elems, dtype=torch.uint8, device=device)
-        q_s = torch.empty(meta_elems, dtype=torch.float16, device=device)
+        q_s = torch.empty(meta_elems, dtype=dtype, device=device)
         q_zp = torch.empty(meta_elems, dtype=torch.uint8, device=device) if has_offsets else None
-        capi.quant(bs, col, w, q_w, q_s, q_zp)
+        capi.quant(bs, col, w, q_w, q_s, q_zp, bf16=bf)
         sets.append((q_w, q_s, q_zp))
         del w
     torch.cuda.synchronize()
-    out = torch.empty(m, n, dtype=torch.float16, device=device)
+    out = torch.empty(m, n, dtype=dtype, device=device)
     return a, sets, out, w_host
 
 
@@ -178,7 +185,7 @@ def bench_gemm(torch, capi, name, device, steps, warmup):
 
     def mk(s):
         q_w, q_s, q_zp = s
-        return lambda: capi.gemm(bs, col, m, n, k, a, q_w, q_s, q_zp, out)
+        return lambda: capi.gemm(bs, col, m, n, k, a, q_w, q_s, q_zp, out, bf16=name in BF16)
 
     launches = [mk(s) for s in sets]
     wall, evt, mode = timed_region(torch, launches, steps, warmup, SETTLE_SECONDS.get(name, 0.0))
@@ -349,7 +356,7 @@ def main(argv=None) -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r,C2r,M128,V128K,B16")
+    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r,C2r,M128,V128K,B16,C4b,C2b")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-context", action="store_true", help="skip the floors and the library comparison")
     args = ap.parse_args(argv)
