@@ -115,7 +115,8 @@ struct Stage {
   static constexpr int kDistance = kStages - 1;  // the slot being refilled is the one nobody reads
 };
 
-template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW>
+// (BF repeats kBF so that the two compilations' kernels carry different names in a trace)
+template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW, bool BF = kBF>
 __global__ __launch_bounds__(64 * (WM * WN + PW))
     __attribute__((amdgpu_waves_per_eu((WM * WN + PW) / 4, (WM * WN + PW) / 4))) void gemm_mfma_kernel(
         const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ S,

@@ -86,7 +86,8 @@ struct Slot {
 // which stay) and for waves that do not split K.
 // ROW: quantization blocks run along N (one k, BS columns); S and Z are then in the packed order
 // described in blkq4_device.h and the lane's column group decides which 64 + 32 bytes it fetches per unit.
-template <int BS, bool HAS_ZP, int DEPTH, int NT, int MT, int kWaves, int AM, bool ROW, bool kRefill, int kSplit>
+// (BF repeats kBF so that the two compilations' kernels carry different names in a trace)
+template <int BS, bool HAS_ZP, int DEPTH, int NT, int MT, int kWaves, int AM, bool ROW, bool kRefill, int kSplit, bool BF = kBF>
 __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t* __restrict__ A,
                                                                const uint4* __restrict__ W,
                                                                const uint16_t* __restrict__ S,
