@@ -117,15 +117,6 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_size_sm80(int block_size, bool colu
 
 namespace {
 
-// bf16 has one blocking, the one the GEMV and GEMM configurations of the fp16 path are quoted on
-bool bf16_blocking_ok(bool bf16, bool column_wise_blocking, std::string* err) {
-  if (bf16 && !column_wise_blocking) {
-    set_error(err, "bf16 is implemented for column-wise blocking only");
-    return false;
-  }
-  return true;
-}
-
 // reference: src/blkq4_f16_gemm_sm80.cu:465-531 and :205-314 (blkq4_quant_sm80_T); bf16: the element type
 // the reference's template anticipates (src/mickey/blk_q4/f16_quant_sm80.cuh:16) and its entry points
 // reject (src/blkq4_f16_gemm_sm80.cu:53)
@@ -134,7 +125,6 @@ int quant_entry(bool bf16, int block_size, bool column_wise_blocking, int rows, 
                 size_t quant_weights_size, void* quant_scales, size_t quant_scales_size, void* offsets,
                 size_t offsets_size, void* err_msg_ptr) {
   auto* err = static_cast<std::string*>(err_msg_ptr);
-  if (!bf16_blocking_ok(bf16, column_wise_blocking, err)) return -1;
   if (!supported_block_size(block_size)) {
     set_error(err, "Unsupported block size: " + std::to_string(block_size));
     return -1;
@@ -242,7 +232,6 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
     return -1;
   }
   const bool has_offsets = offsets_ptr != nullptr && offsets_size > 0;
-  if (!bf16_blocking_ok(bf16, column_wise_blocking, err)) return -1;
 
   if (m <= 0 || n <= 0 || k <= 0) {
     set_error(err, "Empty problem size: " + std::to_string(m) + "x" + std::to_string(n) + "x" +

@@ -125,7 +125,7 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
   return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h)));
 }
 
-// ---- bf16 (blocks along K only) ----------------------------------------------------------------------
+// ---- bf16 ------------------------------------------------------------------------------------------------
 // Dequantized value: bf16( scale * (q - zp) ) with ONE rounding, the same definition as for fp16 with the
 // other 16-bit type.  The nibbles become fp16 pairs (1024 + q) resp. (64 + q) exactly as above; each half is
 // then the fp16 operand of a mixed-precision fma with the scale and -(1024 + zp) * scale resp. -(64 + zp) * scale
@@ -170,6 +170,18 @@ __device__ __forceinline__ bf16x8_t dequant_word_bf16(uint32_t w, const Bf16Cons
   r[6] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p3[0]), c.scale, c.neg_c1));
   r[7] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(p3[1]), c.scale, c.neg_c1));
   return r;
+}
+// Blocks along N: the weights k and k + 1 of a pair have scales of their own (a packed pair of bf16).  d holds
+// q - zp of both, exact in fp16; each product with its scale is exact in fp32 (4 + 8 bits), the packed
+// conversion does the one rounding.  Two instructions for the scales, two multiplies, one conversion.
+__device__ __forceinline__ uint32_t row_pair_bf16(half2_t d, uint32_t scale_pair) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const float s0 = __builtin_bit_cast(float, scale_pair << 16);
+  const float s1 = __builtin_bit_cast(float, scale_pair & 0xffff0000u);
+  bf16x2_t v;
+  v[0] = static_cast<__bf16>(static_cast<float>(d[0]) * s0);
+  v[1] = static_cast<__bf16>(static_cast<float>(d[1]) * s1);
+  return __builtin_bit_cast(uint32_t, v);
 }
 __device__ __forceinline__ bf16x8_t as_bf16x8(uint4 v) {
   uint4_t t = {v.x, v.y, v.z, v.w};

@@ -44,7 +44,7 @@ typedef struct {
   void* scales;        /* fp16 [K/bs][N] */
   void* zero_points;   /* uint8 [K/bs][N] or NULL (symmetric) */
   void* stream;
-  int bf16;            /* 1: src and scales are bf16 (column_wise = 1 only); 0: fp16 */
+  int bf16;            /* 1: src and scales are bf16; 0: fp16 */
 } blkq4_prepack_args;
 
 typedef struct {
@@ -71,8 +71,8 @@ typedef struct {
 int blkq4_dev_prepack(const blkq4_prepack_args* args);
 int blkq4_dev_gemm(const blkq4_gemm_args* args);   /* MFMA tile kernel, every m (made for large m) */
 int blkq4_dev_skinny(const blkq4_gemm_args* args); /* weight-streaming kernel, 1 <= m <= 1024 */
-int blkq4_dev_gemm_bf16(const blkq4_gemm_args* args);   /* the tile kernel with bf16 a, scales, c and bias; column_wise = 1 only */
-int blkq4_dev_skinny_bf16(const blkq4_gemm_args* args); /* the same with bf16 a, scales, c and bias; column_wise = 1 only */
+int blkq4_dev_gemm_bf16(const blkq4_gemm_args* args);   /* the tile kernel with bf16 a, scales, c and bias */
+int blkq4_dev_skinny_bf16(const blkq4_gemm_args* args); /* the same with bf16 a, scales, c and bias */
 int blkq4_dev_repack(const blkq4_repack_args* args);
 const char* blkq4_dev_error_string(int code);
 

@@ -51,7 +51,7 @@
 #include "blkq4_gemm_common.h"
 
 // This file is compiled twice: as it is for fp16, and through blkq4_gemm_bf16.hip, which defines BLKQ4_GEMM_BF16
-// before including it, for bf16 activations, scales and outputs (blocks along K only).
+// before including it, for bf16 activations, scales and outputs.
 #ifdef BLKQ4_GEMM_BF16
 #define BLKQ4_GEMM_ENTRY blkq4_dev_gemm_bf16
 #else
@@ -374,7 +374,7 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   // PM the packed conversion of their results to bf16.
 #define BLKQ4_PIECE_PA(dc_, q_, w_, y_)                                                                       \
   {                                                                                                           \
-    if constexpr (kBF) {                                                                                      \
+    if constexpr (kBF && !ROW) {                                                                              \
       const Bf16Consts& bc_ = (b##dc_)[(y_) / 4][q_];                                                         \
       pf[y_][0] = __builtin_fmaf(static_cast<float>(pt[y_][0]), bc_.scale, (((y_) & 1) == 0) ? bc_.neg_c0 : bc_.neg_c1); \
       pf[y_][1] = __builtin_fmaf(static_cast<float>(pt[y_][1]), bc_.scale, (((y_) & 1) == 0) ? bc_.neg_c0 : bc_.neg_c1); \
@@ -385,11 +385,16 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   }
 #define BLKQ4_PIECE_PM(dst_, dc_, q_, w_, y_)                                                                \
   {                                                                                                          \
-    if constexpr (kBF) {                                                                                     \
+    if constexpr (kBF && !ROW) {                                                                             \
       bf16x2_t v_;                                                                                           \
       v_[0] = static_cast<__bf16>(pf[y_][0]);                                                                \
       v_[1] = static_cast<__bf16>(pf[y_][1]);                                                                \
       wp[dst_][(y_) / 4][(y_) % 4] = __builtin_bit_cast(half2_t, v_);                                        \
+    } else if constexpr (kBF) {                                                                              \
+      /* blocks along N: pt holds q - zp of the pair, each weight has its own bf16 scale */                  \
+      wp[dst_][(y_) / 4][(y_) % 4] = as_half2(row_pair_bf16(                                                 \
+          pt[y_], vec_word(mrow_s[(w_) >> 1][(y_) / 4][(2 * ((y_) % 4) + ((w_)&1)) >> 2],                    \
+                           (2 * ((y_) % 4) + ((w_)&1)) & 3)));                                               \
     } else {                                                                                                 \
       wp[dst_][(y_) / 4][(y_) % 4] =                                                                         \
           pt[y_] * (ROW ? as_half2(vec_word(mrow_s[(w_) >> 1][(y_) / 4][(2 * ((y_) % 4) + ((w_)&1)) >> 2],   \
@@ -601,9 +606,7 @@ int launch_rt(const blkq4_gemm_args* a) {
   const long tiles = static_cast<long>((a->m + 255) / 256) * ((a->n + 255) / 256);
   const long small_tiles = static_cast<long>((a->m + 127) / 128) * ((a->n + 127) / 128);
   const long smallest_tiles = static_cast<long>((a->m + 63) / 64) * ((a->n + 127) / 128);
-  if constexpr (kBF) {
-    if (!a->column_wise) return static_cast<int>(hipErrorInvalidValue);  // bf16: blocks along K only
-  } else if (!a->column_wise) {
+  if (!a->column_wise) {
     // blocks along N (the streaming kernel takes the small row counts)
     if (tiles >= kComputeUnits) return launch_one<BS, HAS_ZP, 8, 2, 1, 4, 0, true>(a);
     if (smallest_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 2, 1, 1, 4, 4, true>(a);

@@ -227,7 +227,7 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
 // rows scale rows (2t, 2t+1, 2t+8, 2t+9) and zero-point rows (2t, 2t+8, 2t+1, 2t+9) sit at
 // positions 4t .. 4t+3.
 // ------------------------------------------------------------------------------------------------
-template <int BS, bool HAS_ZP, bool ALIGNED>
+template <int BS, bool HAS_ZP, bool ALIGNED, bool BF = false>
 __global__ __launch_bounds__(kThreads) void prepack_rowwise_kernel(const uint16_t* __restrict__ src, int K,
                                                                    int N, int ld,
                                                                    uint4* __restrict__ packed_w,
@@ -265,7 +265,7 @@ __global__ __launch_bounds__(kThreads) void prepack_rowwise_kernel(const uint16_
     }
   }
 #define BLKQ4_VALUE(it_, t_) \
-  half_bits_to_float((((t_) >> 1) == 0 ? raw[it_].x : ((t_) >> 1) == 1 ? raw[it_].y : ((t_) >> 1) == 2 ? raw[it_].z : raw[it_].w) >> (16 * ((t_) & 1)) & 0xffffu)
+  bits_to_float<BF>((((t_) >> 1) == 0 ? raw[it_].x : ((t_) >> 1) == 1 ? raw[it_].y : ((t_) >> 1) == 2 ? raw[it_].z : raw[it_].w) >> (16 * ((t_) & 1)) & 0xffffu)
 
 #pragma unroll
   for (int g = 0; g < kGroups; ++g) {
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(kThreads) void prepack_rowwise_kernel(const uint16_
       if constexpr (HAS_ZP) {
         const float rmn = fminf(mn, 0.0f);
         const float rmx = fmaxf(mx, 0.0f);
-        const float scale_f = div_by_15(__fsub_rn(rmx, rmn));
+        const float scale_f = BF ? __fdiv_rn(__fsub_rn(rmx, rmn), 15.0f) : div_by_15(__fsub_rn(rmx, rmn));
         float zero_point_fp = rmn;
         if (scale_f != 0.0f) zero_point_fp = __fsub_rn(0.0f, __fdiv_rn(rmn, scale_f));
         if (zero_point_fp < 0.0f) {
@@ -301,10 +301,10 @@ __global__ __launch_bounds__(kThreads) void prepack_rowwise_kernel(const uint16_
         } else {
           zp = round_0_to_15(zero_point_fp);
         }
-        scale_bits = float_to_half_bits(scale_f);
+        scale_bits = float_to_bits<BF>(scale_f);
       } else {
         const float m = fabsf(mx) > fabsf(mn) ? mx : mn;
-        scale_bits = float_to_half_bits(__fdiv_rn(m, -8.0f));
+        scale_bits = float_to_bits<BF>(__fdiv_rn(m, -8.0f));
         if (m == 0.0f) {
           // all-zero block: the sign comes from the block's first weight (its first column, this k)
           const uint32_t w0 = ((t >> 1) == 0 ? raw[g * kPasses].x : (t >> 1) == 1 ? raw[g * kPasses].y
@@ -314,7 +314,7 @@ __global__ __launch_bounds__(kThreads) void prepack_rowwise_kernel(const uint16_
         }
         zp = 8;
       }
-      const float scale = half_bits_to_float(scale_bits);
+      const float scale = bits_to_float<BF>(scale_bits);
       rs[t] = (scale != 0.0f) ? __fdiv_rn(1.0f, scale) : 0.0f;
       zf[t] = static_cast<float>(zp);
       sbits[t] = scale_bits;
@@ -437,13 +437,19 @@ int launch_prepack_rowwise(const blkq4_prepack_args* a) {
   auto* sc = static_cast<uint16_t*>(a->scales);
   auto* zp = static_cast<uint8_t*>(a->zero_points);
   const bool aligned = (reinterpret_cast<uintptr_t>(a->src) & 15u) == 0 && (a->ld % 8) == 0;
-#define BLKQ4_LAUNCH(ZP_, AL_)                                                                                   \
-  hipLaunchKernelGGL((prepack_rowwise_kernel<BS, ZP_, AL_>), grid, block, 0, stream, src, a->rows, a->columns, \
+#define BLKQ4_LAUNCH(ZP_, AL_, BF_)                                                                                   \
+  hipLaunchKernelGGL((prepack_rowwise_kernel<BS, ZP_, AL_, BF_>), grid, block, 0, stream, src, a->rows, a->columns, \
                      a->ld, pw, sc, zp, k_tiles)
-  if (zp) {
-    if (aligned) BLKQ4_LAUNCH(true, true); else BLKQ4_LAUNCH(true, false);
+  if (a->bf16) {
+    if (zp) {
+      if (aligned) BLKQ4_LAUNCH(true, true, true); else BLKQ4_LAUNCH(true, false, true);
+    } else {
+      if (aligned) BLKQ4_LAUNCH(false, true, true); else BLKQ4_LAUNCH(false, false, true);
+    }
+  } else if (zp) {
+    if (aligned) BLKQ4_LAUNCH(true, true, false); else BLKQ4_LAUNCH(true, false, false);
   } else {
-    if (aligned) BLKQ4_LAUNCH(false, true); else BLKQ4_LAUNCH(false, false);
+    if (aligned) BLKQ4_LAUNCH(false, true, false); else BLKQ4_LAUNCH(false, false, false);
   }
 #undef BLKQ4_LAUNCH
   return static_cast<int>(hipGetLastError());
@@ -451,7 +457,7 @@ int launch_prepack_rowwise(const blkq4_prepack_args* a) {
 
 template <int BS>
 int launch_prepack(const blkq4_prepack_args* a) {
-  if (!a->column_wise) return a->bf16 ? static_cast<int>(hipErrorInvalidValue) : launch_prepack_rowwise<BS>(a);
+  if (!a->column_wise) return launch_prepack_rowwise<BS>(a);
   const unsigned k_tiles = (a->rows + kTileK - 1) / kTileK;
   const dim3 grid(k_tiles * static_cast<unsigned>((a->columns + kTileN - 1) / kTileN));
   const dim3 block(kThreads);

@@ -42,7 +42,7 @@
 #include "blkq4_gemm_common.h"
 
 // This file is compiled twice: as it is for fp16, and through blkq4_skinny_bf16.hip, which defines
-// BLKQ4_SKINNY_BF16 before including it, for bf16 activations, scales and outputs (blocks along K only).
+// BLKQ4_SKINNY_BF16 before including it, for bf16 activations, scales and outputs.
 #ifdef BLKQ4_SKINNY_BF16
 #define BLKQ4_SKINNY_ENTRY blkq4_dev_skinny_bf16
 #else
@@ -344,11 +344,10 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         const uint32_t words[4] = {cur.w[t].x, cur.w[t].y, cur.w[t].z, cur.w[t].w};
-        if constexpr (kBF) {
-          // bf16: blocks along K only
+        if constexpr (kBF && !ROW) {
           Bf16Consts bc[kMeta];
 #pragma unroll
-          for (int q = 0; q < kMeta; ++q) bc[q] = make_bf16_consts(cur.sc[t][ROW ? 0 : q] & okm, cur.zp[t][ROW ? 0 : q]);
+          for (int q = 0; q < kMeta; ++q) bc[q] = make_bf16_consts(cur.sc[t][q] & okm, cur.zp[t][q]);
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const bf16x8_t wf = dequant_word_bf16(words[j], bc[(kMeta == 2) ? (j >> 1) : 0], masks);
@@ -382,10 +381,14 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
               const uint32_t zpair = HAS_ZP ? ((zw[i] >> (8 * hh)) & 0x00ff00ffu) : 0x00080008u;
               const uint32_t src = (i >= 2) ? y : words[j];
               const half2_t s2 = as_half2(sw[2 * i + hh] & okm);
-              if ((i & 1) == 0) {
-                p[i] = (as_half2((src & masks.lo_mask) | masks.magic_1024) + as_half2(0xE400E400u | zpair)) * s2;
+              // q - zp of the pair, exact
+              const half2_t d = ((i & 1) == 0)
+                  ? as_half2((src & masks.lo_mask) | masks.magic_1024) + as_half2(0xE400E400u | zpair)
+                  : as_half2((src & masks.hi_mask) | masks.magic_64) + as_half2(0xD400D400u | (zpair << 4));
+              if constexpr (kBF) {
+                p[i] = as_half2(row_pair_bf16(d, sw[2 * i + hh] & okm));  // a bf16 pair in the same register
               } else {
-                p[i] = (as_half2((src & masks.hi_mask) | masks.magic_64) + as_half2(0xD400D400u | (zpair << 4))) * s2;
+                p[i] = d * s2;
               }
             }
           } else {
@@ -400,7 +403,12 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
           wf[4] = p[2][0]; wf[5] = p[2][1]; wf[6] = p[3][0]; wf[7] = p[3][1];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, as_half8(af[mt][j]), acc[t][mt], 0, 0, 0);
+            if constexpr (kBF) {
+              acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf), as_bf16x8(af[mt][j]),
+                                                                  acc[t][mt], 0, 0, 0);
+            } else {
+              acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, as_half8(af[mt][j]), acc[t][mt], 0, 0, 0);
+            }
           }
         }
       }
@@ -675,17 +683,12 @@ int launch_shape(const blkq4_gemm_args* a) {
 template <int BS>
 int launch_skinny(const blkq4_gemm_args* a) {
   if (a->column_wise) return a->zero_points ? launch_shape<BS, true, false>(a) : launch_shape<BS, false, false>(a);
-  if constexpr (kBF) {
-    return static_cast<int>(hipErrorInvalidValue);
-  } else {
-    return a->zero_points ? launch_shape<BS, true, true>(a) : launch_shape<BS, false, true>(a);
-  }
+  return a->zero_points ? launch_shape<BS, true, true>(a) : launch_shape<BS, false, true>(a);
 }
 
 }  // namespace
 
 extern "C" int BLKQ4_SKINNY_ENTRY(const blkq4_gemm_args* a) {
-  if (kBF && !a->column_wise) return static_cast<int>(hipErrorInvalidValue);  // bf16: blocks along K only
   if (a->m < 1 || a->m > kStreamingMaxRows || (a->n % 16) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
   if (a->n > (1 << 26)) return static_cast<int>(hipErrorInvalidValue);  // a lane's offset inside a slice (up to 8 n rows of 16 bytes) is 32 bits wide
   if (!a->column_wise) {

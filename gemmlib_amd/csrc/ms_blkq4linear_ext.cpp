@@ -6,7 +6,7 @@
 // Differences on purpose: kernels run on torch's current stream instead of the default stream, a
 // scale-only quantization returns an empty uint8 tensor for q_zp (the reference returns an undefined
 // tensor that its own forward() cannot take), and bfloat16 weights / inputs are taken too (scales, bias and
-// output then are bfloat16; blocks along K only), through blkq4_bf16_quant_sm80 / blkq4_bf16_gemm_sm80.
+// output then are bfloat16), through blkq4_bf16_quant_sm80 / blkq4_bf16_gemm_sm80.
 
 #include <torch/extension.h>
 

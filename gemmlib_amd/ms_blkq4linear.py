@@ -15,7 +15,7 @@ them, and takes 2-D inputs only):
   the module's extra state, so ``state_dict()`` / ``load_state_dict()`` round-trip a quantized layer;
   ``BlkQ4Linear.from_packed`` builds a layer straight from packed tensors, without the fp16 weights;
 * ``forward`` accepts any number of leading dimensions (``[..., in_features]``);
-* bfloat16 weights make a bfloat16 layer (bfloat16 scales, inputs, bias and outputs; ``col_wise=True`` only).
+* bfloat16 weights make a bfloat16 layer (bfloat16 scales, inputs, bias and outputs).
 """
 
 import torch

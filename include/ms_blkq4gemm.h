@@ -136,8 +136,8 @@ int blkq4_fp16_repack_sm80(
  * 16-bit buffer holding bf16; buffer sizes from blkq4_fp16_quant_size_sm80.  Arithmetic: the reference
  * quantizer's with the scale rounded to bf16; weight = bf16(scale * (q - offset)) with one rounding; fp32
  * accumulation, one rounding of the output to bf16, then the bias added in fp32 and rounded to bf16.
- * Column-wise blocking only (column_wise_blocking = false fails with a message).  The packed weights
- * and the offsets are interchangeable with the fp16 entry points'; the scales are not.
+ * Both blockings.  The packed weights and the offsets are interchangeable with the fp16 entry points';
+ * the scales are not.
  */
 int blkq4_bf16_quant_sm80(
     int block_size,

@@ -1,8 +1,8 @@
 """GPU parity of the bf16 entry points (blkq4_bf16_quant_sm80, blkq4_bf16_gemm_sm80), through the C ABI.
 
 Bars:
-  * quantizer: bit-exact against the oracle (nibbles in the library's order, scales, zero-points), on the
-    bf16-exact known-answer construction and on Gaussian data, ragged and strided sources included;
+  * quantizer, both blockings: bit-exact against the oracle (nibbles in the library's order, scales, zero-points),
+    on the bf16-exact known-answer construction and on Gaussian data, ragged and strided sources included;
   * GEMM on the known-answer construction with activations on the 0.25 grid (the reference's own
     exact-equality test, test/blkq4_fp16_gemm_sm80_test.cu:194-256,469-472, with the element type changed):
     every partial sum is exact in fp32, so the output is BIT-EXACT whatever the summation order;
@@ -32,35 +32,40 @@ def dev_to_bits(t: torch.Tensor) -> np.ndarray:
     return t.view(torch.int16).cpu().numpy().view(np.uint16)
 
 
-def quantize_bf16(capi, device, bs, weights_bits, has_offsets, w_dev=None, rows=None, columns=None, ld=None):
+def quantize_bf16(capi, device, bs, weights_bits, has_offsets, w_dev=None, rows=None, columns=None, ld=None, col=True):
     n, k = weights_bits.shape if columns is None else (columns, rows)
-    w_elems, meta_elems = capi.quant_size(bs, True, k, n)
+    w_elems, meta_elems = capi.quant_size(bs, col, k, n)
     if w_dev is None:
         w_dev = bits_to_dev(weights_bits, device)
     q_w = torch.full((w_elems,), 0xA5, dtype=torch.uint8, device=device)
     q_s = torch.full((meta_elems,), float("nan"), dtype=torch.bfloat16, device=device)
     q_zp = torch.full((meta_elems,), 0xEE, dtype=torch.uint8, device=device) if has_offsets else None
-    capi.quant(bs, True, w_dev, q_w, q_s, q_zp, bf16=True, rows=rows, columns=columns, ld=ld)
+    capi.quant(bs, col, w_dev, q_w, q_s, q_zp, bf16=True, rows=rows, columns=columns, ld=ld)
     torch.cuda.synchronize()
     return q_w, q_s, q_zp
 
 
-def gemm_bf16(capi, device, bs, a_bits, q_w, q_s, q_zp, n, bias=None):
+def gemm_bf16(capi, device, bs, a_bits, q_w, q_s, q_zp, n, bias=None, col=True):
     m, k = a_bits.shape
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=device)
-    capi.gemm(bs, True, m, n, k, bits_to_dev(a_bits, device), q_w, q_s, q_zp, out, bias=bias, bf16=True)
+    capi.gemm(bs, col, m, n, k, bits_to_dev(a_bits, device), q_w, q_s, q_zp, out, bias=bias, bf16=True)
     torch.cuda.synchronize()
     assert not torch.isnan(out).any()
     return dev_to_bits(out)
 
 
-def check_quantizer(oracle, capi, device, bs, weights_bits, has_offsets, **kw):
+def check_quantizer(oracle, capi, device, bs, weights_bits, has_offsets, col=True, **kw):
     n, k = weights_bits.shape
-    q_w, q_s, q_zp = quantize_bf16(capi, device, bs, weights_bits, has_offsets, **kw)
-    canon, s, z = oracle.quantize(bs, True, weights_bits, has_offsets, bf16=True)
-    assert np.array_equal(dev_to_bits(q_s).reshape(k // bs, n), s.T), "scales differ"
+    q_w, q_s, q_zp = quantize_bf16(capi, device, bs, weights_bits, has_offsets, col=col, **kw)
+    canon, s, z = oracle.quantize(bs, col, weights_bits, has_offsets, bf16=True)
+    # scales and zero-points in the order the reference's entry point returns them (blocks along K: row-major
+    # [K/bs, N]; blocks along N: its 16-row rearrangement), which is a matter of 16-bit patterns only
+    ps, pz = oracle.prepack_meta_sm80(bs, col, k, n, s, z)
+    assert np.array_equal(dev_to_bits(q_s), ps.view(np.uint16)), "scales differ"
+    if col:
+        assert np.array_equal(ps.view(np.uint16).reshape(k // bs, n), s.T)
     if has_offsets:
-        assert np.array_equal(q_zp.cpu().numpy().reshape(k // bs, n), z.T), "zero-points differ"
+        assert np.array_equal(q_zp.cpu().numpy(), pz), "zero-points differ"
     got_w = q_w.cpu().numpy()
     want = oracle.native_from_canonical(canon)
     if not np.array_equal(got_w, want):
@@ -229,13 +234,91 @@ def test_module_takes_bfloat16(oracle, capi, device, scale_only, m):
     y = layer(x.to(device))
     assert y.shape == (3, m, n) and y.dtype == torch.bfloat16
     w_bits = w.view(torch.int16).numpy().view(np.uint16)
-    canon, s, z = oracle.quantize(bs, True, w_bits, not scale_only, bf16=True)
+    canon, _, _ = oracle.quantize(bs, True, w_bits, not scale_only, bf16=True)
     assert np.array_equal(layer.q_weights.cpu().numpy(), oracle.native_from_canonical(canon))
     x_bits = x.reshape(3 * m, k).view(torch.int16).numpy().view(np.uint16)
-    ref = oracle.gemm(x_bits, oracle.dequantize(bs, True, canon, s, z, bf16=True), bf16=True)
-    ref = torch.from_numpy(ref.view(np.int16)).view(torch.bfloat16) + bias
-    assert max_rel_err(y.reshape(3 * m, n).float().cpu().numpy(), ref.float().numpy()) <= TOLERANCE
+
+    def check(out, col):
+        """against the oracle's GEMM plus the bias: an output's error is measured against the larger of the two
+        summands (the sum itself may cancel), as a separate add of two bf16 tensors would be"""
+        canon, s, z = oracle.quantize(bs, col, w_bits, not scale_only, bf16=True)
+        c = oracle.gemm(x_bits, oracle.dequantize(bs, col, canon, s, z, bf16=True), bf16=True)
+        c = torch.from_numpy(c.view(np.int16)).view(torch.bfloat16)
+        ref = (c + bias).float().numpy()
+        scale = np.maximum(np.maximum(np.abs(c.float().numpy()), np.abs(bias.float().numpy())[None, :]), 1e-3)
+        got = out.reshape(3 * m, n).float().cpu().numpy()
+        # a unit in the last place of the GEMM output (2^-7) plus the rounding of the sum (2^-8 of up to twice the scale)
+        assert np.max(np.abs(got - ref) / scale) <= 2 * TOLERANCE
+
+    check(y, True)
     with pytest.raises(RuntimeError, match="must have the input's element type"):
         layer(x.to(device).to(torch.float16))
-    with pytest.raises(RuntimeError, match="column-wise blocking only"):
-        mod.BlkQ4Linear(bs, False, scale_only, w.to(device))
+    # blocks along N through the module
+    row_layer = mod.BlkQ4Linear(bs, False, scale_only, w.to(device), bias.to(device))
+    check(row_layer(x.to(device)), False)
+
+
+# ---------------------------------------------------------------------------------------------
+# blocks along N (column_wise_blocking = false)
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("bs", [16, 32, 64])
+@pytest.mark.parametrize("has_offsets", [True, False])
+@pytest.mark.parametrize("rows,columns", [(64, 64), (128, 192), (576, 704)])
+def test_row_wise_quantizer_gives_back_the_known_answers(oracle, capi, device, bs, has_offsets, rows, columns):
+    kat = bf16_kat(oracle, bs, rows, columns, has_offsets, seed=rows + columns + bs, column_wise=False)
+    _, _, _, canon, s, z = check_quantizer(oracle, capi, device, bs, kat["weights"], has_offsets, col=False)
+    assert np.array_equal(canon, kat["canon_w"]) and np.array_equal(s, kat["scales"])
+    if has_offsets:
+        assert np.array_equal(z, kat["zps"])
+
+
+@pytest.mark.parametrize("bs,has_offsets,rows,columns", [(16, True, 512, 352), (32, False, 1024, 1024), (64, True, 448, 832)])
+def test_row_wise_quantizer_on_gaussian_weights(oracle, capi, device, bs, has_offsets, rows, columns):
+    _, w = gaussian_bits(oracle, rows + columns + 1, 1, columns, rows)
+    check_quantizer(oracle, capi, device, bs, w, has_offsets, col=False)
+
+
+# the reference's row-wise cases (test/blkq4_fp16_gemm_sm80_test.cu:480-499,508-512), M = 1 and ragged M, the tile
+# kernel's four tile shapes, very wide N in the streaming kernel
+ROW_WISE_EXACT_CASES = [
+    (32, False, 32, 32, 64), (32, True, 32, 96, 192), (32, True, 256, 672, 576), (32, False, 512, 2048 + 32, 960),
+    (16, True, 256, 672, 576), (64, False, 256, 1024, 576), (16, False, 16, 704, 576), (64, True, 16, 1024, 576),
+    (64, False, 1, 1024, 576), (16, True, 2, 160, 128), (64, True, 7, 1088, 192), (32, True, 17, 96, 192),
+    (16, True, 65, 544, 256), (64, True, 129, 1088, 576), (16, True, 400, 672, 576), (32, True, 1000, 4128, 128),
+    (64, True, 640, 4160, 192), (16, True, 4096, 4096, 128), (64, True, 4096, 4096, 192), (32, True, 160, 96, 8256),
+    (64, False, 1, 14336, 4096), (32, True, 2, 16384, 2112), (16, True, 8, 28672, 1088), (64, True, 16, 16384, 8256),
+]
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", ROW_WISE_EXACT_CASES)
+def test_row_wise_gemm_exact_on_known_answer_construction(oracle, capi, device, bs, has_offsets, m, n, k):
+    rng = np.random.default_rng(m * 131 + n * 17 + k + bs + has_offsets)
+    kat = bf16_kat(oracle, bs, k, n, has_offsets, seed=m + n + k, column_wise=False)
+    a = grid_activations_bf16(oracle, rng, m, k)
+    q_w, q_s, q_zp = quantize_bf16(capi, device, bs, kat["weights"], has_offsets, col=False)
+    assert np.array_equal(q_w.cpu().numpy(), oracle.native_from_canonical(kat["canon_w"]))
+    got = gemm_bf16(capi, device, bs, a, q_w, q_s, q_zp, n, col=False)
+    c64 = oracle.bf16_to_f32(a).astype(np.float64) @ kat["exact"].T
+    assert np.array_equal(c64.astype(np.float32).astype(np.float64), c64)   # the sums fit a float
+    ref = oracle.gemm(a, kat["weights"], bf16=True)
+    assert np.array_equal(ref, oracle.f32_to_bf16(c64.astype(np.float32)))
+    if not np.array_equal(got, ref):
+        bad = np.argwhere(got != ref)
+        raise AssertionError(f"{bad.shape[0]} of {m * n} outputs differ, first {bad[:5].tolist()}: "
+                             f"got {got[tuple(bad[0])]:#06x} want {ref[tuple(bad[0])]:#06x}")
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k,seed", [
+    (32, True, 64, 1024, 1024, 3235), (64, False, 1, 4096, 4096, 3236), (16, True, 16, 2816, 1024, 3237),
+    (64, True, 200, 1152, 512, 3238), (64, True, 2048, 4096, 1024, 3239),
+])
+def test_row_wise_gemm_on_gaussian_data(oracle, capi, device, bs, has_offsets, m, n, k, seed):
+    a, w = gaussian_bits(oracle, seed, m, n, k)
+    q_w, q_s, q_zp, canon, s, z = check_quantizer(oracle, capi, device, bs, w, has_offsets, col=False)
+    got = gemm_bf16(capi, device, bs, a, q_w, q_s, q_zp, n, col=False)
+    ref = oracle.gemm(a, oracle.dequantize(bs, False, canon, s, z, bf16=True), bf16=True)
+    err = max_rel_err(oracle.bf16_to_f32(got), oracle.bf16_to_f32(ref))
+    print(f"bf16 row-wise m={m} n={n} k={k} bs={bs} zp={has_offsets}: max rel err {err:.3e}, "
+          f"bit-identical outputs {float(np.mean(got == ref)):.4f}")
+    assert err <= TOLERANCE

@@ -69,19 +69,20 @@ def test_float_to_bf16_rounding(oracle):
 
 @pytest.mark.parametrize("bs", [16, 32, 64])
 @pytest.mark.parametrize("has_offsets", [False, True])
-@pytest.mark.parametrize("rows,cols", [(64, 32), (128, 96), (256, 160)])
-def test_quantizer_round_trip_on_bf16_exact_data(oracle, bs, has_offsets, rows, cols):
-    kat = bf16_kat(oracle, bs, rows, cols, has_offsets, seed=rows + cols + bs)
+@pytest.mark.parametrize("rows,cols", [(64, 64), (128, 192), (256, 320)])
+@pytest.mark.parametrize("col", [True, False])
+def test_quantizer_round_trip_on_bf16_exact_data(oracle, bs, has_offsets, rows, cols, col):
+    kat = bf16_kat(oracle, bs, rows, cols, has_offsets, seed=rows + cols + bs, column_wise=col)
     # the construction is exact: float64 product equals the bf16 weight
     w64 = oracle.bf16_to_f32(kat["weights"]).astype(np.float64)
     assert np.array_equal(w64, kat["exact"])
-    cw, s, z = oracle.quantize(bs, True, kat["weights"], has_offsets, bf16=True)
+    cw, s, z = oracle.quantize(bs, col, kat["weights"], has_offsets, bf16=True)
     assert np.array_equal(cw, kat["canon_w"])
     assert np.array_equal(s, kat["scales"])
     if has_offsets:
         assert np.array_equal(z, kat["zps"])
     # and back: the oracle's dequantization reproduces the weights bit for bit
-    assert np.array_equal(oracle.dequantize(bs, True, cw, s, z, bf16=True), kat["weights"])
+    assert np.array_equal(oracle.dequantize(bs, col, cw, s, z, bf16=True), kat["weights"])
 
 
 def test_quantizer_scale_is_rounded_to_bf16_not_fp16(oracle):
@@ -144,7 +145,7 @@ def _buf(nbytes, address=0x1000):
 
 
 @pytest.mark.parametrize("kwargs,message", [
-    (dict(col=False), "bf16 is implemented for column-wise blocking only"),
+    (dict(col=False, bs=64, n=96, s=_buf(64 * 1 * 2), c=_buf(4 * 96 * 2)), "Kernel execution failed: Error Invalid Problem"),
     (dict(bs=8), "Unsupported block size: 8"),
     (dict(m=0), "Empty problem size: 0x64x64"),
     (dict(a=_buf(10)), "Unexpected activation tensor size: 10 expected: 512"),
@@ -177,7 +178,7 @@ def test_bf16_quant_validation_messages(capi):
         finally:
             lib.blkq4_error_message_destroy(err)
 
-    assert call(col=False) == (-1, "bf16 is implemented for column-wise blocking only")
+    assert call(col=False, qs_bytes=60 * 2) == (-1, "Unexpected scale tensor size: 60 expected: 64")
     assert call(bs=128) == (-1, "Unsupported block size: 128")
     assert call(rows=100) == (-1, "Cannot block quantize matrix with rows: 100")
     assert call(qs_bytes=100) == (-1, "Unexpected scale tensor size: 50 expected: 64")
