@@ -72,16 +72,19 @@ DESCRIPTION = {
 # read these counters for itself; the figures are refreshed when a kernel changes.
 COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65552.0, "WRITE_SIZE": 1.0}
 COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
-    "C4": (44090.8, 16384.0),
-    "C2": (4416.4, 8.0),
-    "C3": (13863.8, 344.0),
-    "C5": (860310.0, 229376.0),
-    "C5_prepack": (229442.0, 158472.6),
-    "C4r": (44090.6, 16384.0),
-    "C2r": (4408.9, 8.0),
+    "C4": (44106.8, 16384.0),
+    "C2": (4416.0, 8.0),
+    "C3": (13870.4, 344.0),
+    "C5": (860484.2, 229376.0),
+    "C5_prepack": (229445.4, 158478.8),
+    "C4r": (44108.3, 16384.0),
+    "C2r": (4417.4, 8.0),
     "C1": (865.1, 128.0),
-    "M128": (8654.0, 1024.0),
-    "V128K": (136416.0, 250.7),
+    "M128": (8653.7, 1024.0),
+    "V128K": (136437.3, 250.7),
+    "B16": (63847.2, 896.0),
+    "C4b": (44121.8, 16384.0),
+    "C2b": (4418.8, 8.0),
 }
 
 
