@@ -14,33 +14,40 @@ from gpu_util import to_np
 
 pytestmark = pytest.mark.gpu
 
-# (block_size, column_wise, has_offsets, m, n, k): tile kernel, streaming kernel (whole rows in LDS, rows per
-# slot, row groups), row-wise streaming and row-wise tile kernel
+# (block_size, column_wise, has_offsets, m, n, k, bf16): tile kernel, streaming kernel (whole rows in LDS, rows per
+# slot, row groups), row-wise streaming and row-wise tile kernel; then the bf16 entry points on both kernels
 SHAPES = [
-    (64, True, True, 300, 512, 256), (32, True, False, 1, 256, 512), (16, True, True, 16, 64, 8256),
-    (64, True, True, 96, 256, 512), (32, False, True, 8, 128, 256), (64, False, False, 500, 256, 128),
+    (64, True, True, 300, 512, 256, False), (32, True, False, 1, 256, 512, False), (16, True, True, 16, 64, 8256, False),
+    (64, True, True, 96, 256, 512, False), (32, False, True, 8, 128, 256, False), (64, False, False, 500, 256, 128, False),
+    (32, True, True, 4, 256, 512, True), (64, True, False, 16, 64, 8256, True), (64, True, True, 300, 512, 256, True),
+    (32, False, True, 8, 128, 256, True),
 ]
 
 
-def _problem(capi, device, bs, col, zp, m, n, k, seed):
+def _problem(capi, device, bs, col, zp, m, n, k, bf, seed):
+    dtype = torch.bfloat16 if bf else torch.float16
     g = torch.Generator(device="cpu").manual_seed(seed)
-    w = (torch.randn(n, k, generator=g) * 0.02).to(torch.float16).to(device)
-    a = torch.randn(m, k, generator=g).to(torch.float16).to(device)
+    w = (torch.randn(n, k, generator=g) * 0.02).to(dtype).to(device)
+    a = torch.randn(m, k, generator=g).to(dtype).to(device)
     w_elems, meta_elems = capi.quant_size(bs, col, k, n)
     q_w = torch.empty(w_elems, dtype=torch.uint8, device=device)
-    q_s = torch.empty(meta_elems, dtype=torch.float16, device=device)
+    q_s = torch.empty(meta_elems, dtype=dtype, device=device)
     q_z = torch.empty(meta_elems, dtype=torch.uint8, device=device) if zp else None
-    out = torch.zeros(m, n, dtype=torch.float16, device=device)
+    out = torch.zeros(m, n, dtype=dtype, device=device)
     return w, a, q_w, q_s, q_z, out
+
+
+def _bits(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
 
 
 def _capture_and_replay(capi, device, warm):
     problems = [_problem(capi, device, *s, seed=50 + i) for i, s in enumerate(SHAPES)]
 
     def enqueue():
-        for (bs, col, zp, m, n, k), (w, a, q_w, q_s, q_z, out) in zip(SHAPES, problems):
-            capi.quant(bs, col, w, q_w, q_s, q_z)
-            capi.gemm(bs, col, m, n, k, a, q_w, q_s, q_z, out)
+        for (bs, col, zp, m, n, k, bf), (w, a, q_w, q_s, q_z, out) in zip(SHAPES, problems):
+            capi.quant(bs, col, w, q_w, q_s, q_z, bf16=bf)
+            capi.gemm(bs, col, m, n, k, a, q_w, q_s, q_z, out, bf16=bf)
 
     if warm:
         enqueue()
@@ -60,7 +67,7 @@ def _capture_and_replay(capi, device, warm):
             w.add_(0.001 * (replay + 1))
         enqueue()
         torch.cuda.synchronize()
-        want = [to_np(p[5]).copy() for p in problems]
+        want = [_bits(p[5]).copy() for p in problems]
         want_w = [to_np(p[2]).copy() for p in problems]
         for p in problems:
             p[5].fill_(float("nan"))
@@ -70,7 +77,7 @@ def _capture_and_replay(capi, device, warm):
         torch.cuda.synchronize()
         for s, p, c, qw in zip(SHAPES, problems, want, want_w):
             assert np.array_equal(to_np(p[2]), qw), f"replay {replay}: packed weights differ for {s}"
-            assert np.array_equal(to_np(p[5]).view(np.uint16), c.view(np.uint16)), f"replay {replay}: output differs for {s}"
+            assert np.array_equal(_bits(p[5]), c), f"replay {replay}: output differs for {s}"
 
 
 def test_replays_match_eager(capi, device):
