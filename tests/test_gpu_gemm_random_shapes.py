@@ -73,3 +73,33 @@ def test_random_shape(oracle, capi, device, bs, has_offsets, col, m, n, k, with_
         torch.cuda.synchronize()
         out += bias
         assert torch.equal(fused.view(torch.int16), out.view(torch.int16))
+
+
+@pytest.mark.parametrize("bs,has_offsets,col,m,n,k,with_bias", draw_cases())
+def test_random_shape_bf16(oracle, capi, device, bs, has_offsets, col, m, n, k, with_bias):
+    """the same shapes through blkq4_bf16_quant_sm80 / blkq4_bf16_gemm_sm80: quantizer bit-exact, GEMM within the
+    same bound (a bf16 output's unit in the last place is up to 2^-7 = 0.8e-2 of its value)"""
+    from test_gpu_bf16 import bits_to_dev, dev_to_bits, gaussian_bits, quantize_bf16
+    a, w = gaussian_bits(oracle, m * 7 + n * 3 + k, m, n, k)
+    q_w, q_s, q_zp = quantize_bf16(capi, device, bs, w, has_offsets, col=col)
+    canon, s, z = oracle.quantize(bs, col, w, has_offsets, bf16=True)
+    assert np.array_equal(q_w.cpu().numpy(), oracle.native_from_canonical(canon))
+    ps, pz = oracle.prepack_meta_sm80(bs, col, k, n, s, z)
+    assert np.array_equal(dev_to_bits(q_s), ps.view(np.uint16))
+    a_dev = bits_to_dev(a, device)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=device)
+    capi.gemm(bs, col, m, n, k, a_dev, q_w, q_s, q_zp, out, bf16=True)
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()
+    got = oracle.bf16_to_f32(dev_to_bits(out))
+    rows = np.arange(m) if m * n * k <= 3e9 else np.unique(np.concatenate([[0, m - 1], np.arange(0, m, max(1, m // 64))]))
+    ref = oracle.gemm(np.ascontiguousarray(a[rows]), oracle.dequantize(bs, col, canon, s, z, bf16=True), bf16=True)
+    assert max_rel_err(got[rows], oracle.bf16_to_f32(ref)) <= TOLERANCE
+    if with_bias:
+        g = torch.Generator(device="cpu").manual_seed(n + k)
+        bias = (torch.randn(n, generator=g) * 0.25).to(torch.bfloat16).to(device)
+        fused = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=device)
+        capi.gemm(bs, col, m, n, k, a_dev, q_w, q_s, q_zp, fused, bias=bias, bf16=True)
+        torch.cuda.synchronize()
+        out += bias
+        assert torch.equal(fused.view(torch.int16), out.view(torch.int16))
