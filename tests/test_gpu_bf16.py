@@ -104,16 +104,21 @@ def test_quantizer_on_values_outside_fp16(oracle, capi, device):
     """magnitudes from 1e-30 to 1e30 per block (a bf16 has the exponent range of a float), zeros of both signs,
     all-zero blocks"""
     rng = np.random.default_rng(3)
-    n, k = 96, 512
+    n, k = 128, 512
     mag = 10.0 ** rng.integers(-30, 31, (n, k // 16)).astype(np.float64)
     w = (rng.standard_normal((n, k)) * np.repeat(mag, 16, axis=1)).astype(np.float32)
     w[5, 64:128] = 0.0
     w[6, 0:64] = -0.0
     w[7, 128:192] = np.abs(w[7, 128:192])          # a block of one sign
+    w[8, 192:256] = 3.0e38                           # a range that overflows a float: the scale is infinite
+    w[8, 200] = -3.0e38
+    w[9, 256:320] = 2.0 ** -133                      # bf16 subnormals
+    w[9, 300] = -3 * 2.0 ** -133
     bits = oracle.f32_to_bf16(w)
     for bs in (16, 32, 64):
         for has_offsets in (True, False):
-            check_quantizer(oracle, capi, device, bs, bits, has_offsets)
+            for col in (True, False):
+                check_quantizer(oracle, capi, device, bs, bits, has_offsets, col=col)
 
 
 def test_quantizer_on_strided_and_unaligned_source(oracle, capi, device):
