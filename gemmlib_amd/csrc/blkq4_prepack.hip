@@ -51,6 +51,16 @@ __device__ __forceinline__ float div_by_15(float x) {
   return __fmaf_rn(r, y, q);
 }
 
+// source and packed weights are touched once per launch: non-temporal requests
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_once_16(const void* p) {
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store_once_16(void* p, const uint4& v) {
+  __builtin_nontemporal_store(u32x4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4_t*>(p));
+}
+
 // nibble position of weight t (0..7) inside its 32-bit word
 __device__ __forceinline__ constexpr int nibble_shift(int t) { return 4 * ((t >> 1) + 4 * (t & 1)); }
 
@@ -97,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
     if (k_ok && n < N) {
       const uint16_t* p = src + static_cast<size_t>(n) * ld + (k0 + kl);
       if constexpr (ALIGNED) {
-        raw[it] = *reinterpret_cast<const uint4*>(p);
+        raw[it] = load_once_16(p);
       } else {
         uint32_t w[4];
 #pragma unroll
@@ -195,7 +205,7 @@ __global__ __launch_bounds__(kThreads) void prepack_kernel(const uint16_t* __res
     const int n = n0 + nl;
     if (k < K && n < N) {
       const uint4 val = *reinterpret_cast<const uint4*>(&w_lds[ksl][nl][0]);
-      packed_w[static_cast<size_t>(k >> 5) * N + n] = val;
+      store_once_16(&packed_w[static_cast<size_t>(k >> 5) * N + n], val);
     }
   }
   // scales / zero-points: row-major [K/BS][N]
@@ -255,7 +265,7 @@ __global__ __launch_bounds__(kThreads) void prepack_rowwise_kernel(const uint16_
     if (k_ok && n < N) {  // N is a multiple of BS: a block is all in or all out
       const uint16_t* p = src + static_cast<size_t>(n) * ld + (k0 + kl);
       if constexpr (ALIGNED) {
-        raw[it] = *reinterpret_cast<const uint4*>(p);
+        raw[it] = load_once_16(p);
       } else {
         uint32_t w[4];
 #pragma unroll
@@ -362,7 +372,7 @@ __global__ __launch_bounds__(kThreads) void prepack_rowwise_kernel(const uint16_
     const int n = n0 + nl;
     if (k < K && n < N) {
       const uint4 val = *reinterpret_cast<const uint4*>(&w_lds[ksl][nl][0]);
-      packed_w[static_cast<size_t>(k >> 5) * N + n] = val;
+      store_once_16(&packed_w[static_cast<size_t>(k >> 5) * N + n], val);
     }
   }
 }

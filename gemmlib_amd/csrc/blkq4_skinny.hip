@@ -53,6 +53,16 @@ namespace {
 
 using namespace blkq4;
 
+// the packed weights are read once per launch
+#ifdef BLKQ4_W_TEMPORAL
+__device__ __forceinline__ uint4 BLKQ4_W_LOAD(const uint4_t* p) { const uint4_t v = *p; return make_uint4(v[0], v[1], v[2], v[3]); }
+#else
+__device__ __forceinline__ uint4 BLKQ4_W_LOAD(const uint4_t* p) {
+  const uint4_t v = __builtin_nontemporal_load(p);
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+#endif
+
 #ifdef BLKQ4_SKINNY_BF16
 constexpr bool kBF = true;
 #else
@@ -224,7 +234,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       const int tile_ = ((cg_) * kTileWaves + wt) * NT + t;                                    \
       const int tu_ = (tile_ < tiles) ? tile_ : (cg_) * (kTileWaves * NT);                     \
       const size_t wu_ = ((static_cast<size_t>(4 * sl_) * N + tu_ * 16) * 16) & keep64_;       \
-      (dst_).w[t] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(W) + wu_ + wl_); \
+      (dst_).w[t] = BLKQ4_W_LOAD(reinterpret_cast<const uint4_t*>(reinterpret_cast<const char*>(W) + wu_ + wl_)); \
       if (ROW) {                                                                               \
         const size_t mu_ = (static_cast<size_t>(tu_ * 16 / BS) * K + sl_ * 128) & keep64_;     \
         const char* sp_ = reinterpret_cast<const char*>(S) + mu_ * 2 + ml_ * 2;                \
