@@ -573,7 +573,9 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
                          add_bias_pair_t<kBF>(v.z, bias8.z), add_bias_pair_t<kBF>(v.w, bias8.w));
         }
         const int m = m0 + wm * (32 * RT) + r0 * 32 + row;
-        if (m < M && col < N) *reinterpret_cast<uint4*>(C + static_cast<size_t>(m) * N + col) = v;
+        if (m < M && col < N) {  // written once, not read again by this launch
+          __builtin_nontemporal_store(uint4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<uint4_t*>(C + static_cast<size_t>(m) * N + col));
+        }
       }
     }
   }
