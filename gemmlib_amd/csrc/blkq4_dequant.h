@@ -173,14 +173,16 @@ __device__ __forceinline__ bf16x8_t dequant_word_bf16(uint32_t w, const Bf16Cons
 }
 // Blocks along N: the weights k and k + 1 of a pair have scales of their own (a packed pair of bf16).  d holds
 // q - zp of both, exact in fp16; each product with its scale is exact in fp32 (4 + 8 bits), the packed
-// conversion does the one rounding.  Two instructions for the scales, two multiplies, one conversion.
+// conversion does the one rounding.  Two instructions for the scales, two mixed-precision fmas, one conversion.
 __device__ __forceinline__ uint32_t row_pair_bf16(half2_t d, uint32_t scale_pair) {
   typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
   const float s0 = __builtin_bit_cast(float, scale_pair << 16);
   const float s1 = __builtin_bit_cast(float, scale_pair & 0xffff0000u);
   bf16x2_t v;
-  v[0] = static_cast<__bf16>(static_cast<float>(d[0]) * s0);
-  v[1] = static_cast<__bf16>(static_cast<float>(d[1]) * s1);
+  // (written as fmas with a zero addend: one v_fma_mix_f32 per weight, where a conversion and a multiply would be two;
+  // a zero weight comes out as +0 whatever the scale's sign, which no sum can tell from -0)
+  v[0] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(d[0]), s0, 0.0f));
+  v[1] = static_cast<__bf16>(__builtin_fmaf(static_cast<float>(d[1]), s1, 0.0f));
   return __builtin_bit_cast(uint32_t, v);
 }
 __device__ __forceinline__ bf16x8_t as_bf16x8(uint4 v) {
