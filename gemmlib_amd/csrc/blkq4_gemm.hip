@@ -135,6 +135,9 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   constexpr int kBM = 32 * RT * WM;
   constexpr int kMeta = (BS == 16) ? 2 : 1;  // quantization blocks inside a lane's 32-deep unit
   constexpr int kMfmas = RT * NT;            // MFMAs of one 16-deep k step
+  // 32-row tiles, and 64-row tiles of eight waves, are launched for problems of one row tile only: every packed
+  // weight is then read once per launch
+  constexpr bool kWeightsOnce = RT == 1 || (RT == 2 && WN == 8);
   static_assert(kStages * St::kBytes <= 160 * 1024, "LDS ring does not fit");
   static_assert(NT == 1 || NT == 2, "the scale / zero-point copy covers at most two fragments");
   __shared__ __attribute__((aligned(1024))) uint8_t lds[kStages * St::kBytes];
@@ -240,7 +243,11 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
                     a_off[(q_) < kAOps ? (q_) : 0]);                                                      \
     } else if ((q_) < kAOps + kBOps) {                                                                    \
       const int p_ = ((q_) >= kAOps && (q_) < kAOps + kBOps) ? (q_) - kAOps : 0;                           \
-      async_copy_16(sbase_ + b_dst[p_], W + static_cast<size_t>(tile_) * b_stride, b_off[p_]);            \
+      if constexpr (kWeightsOnce) {                                                                       \
+        async_copy_16_once(sbase_ + b_dst[p_], W + static_cast<size_t>(tile_) * b_stride, b_off[p_]);     \
+      } else {                                                                                            \
+        async_copy_16(sbase_ + b_dst[p_], W + static_cast<size_t>(tile_) * b_stride, b_off[p_]);          \
+      }                                                                                                   \
     } else {                                                                                              \
       const int p_ = ((q_) >= kAOps + kBOps) ? (q_) - kAOps - kBOps : 0;                                   \
       async_copy_4_flat(sbase_ + meta_dst[p_], meta_ptr[p_] + static_cast<size_t>(tile_) * meta_step[p_]); \

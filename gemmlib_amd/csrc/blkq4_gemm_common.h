@@ -15,6 +15,11 @@ __device__ __forceinline__ void async_copy_16(uint32_t lds_base, const void* bas
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base)
                : "memory");
 }
+// the same with the non-temporal hint, for data that this launch reads once
+__device__ __forceinline__ void async_copy_16_once(uint32_t lds_base, const void* base, uint32_t offset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_base), "v"(offset), "s"(base)
+               : "memory");
+}
 __device__ __forceinline__ void async_copy_4_flat(uint32_t lds_base, const void* gptr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
 }
