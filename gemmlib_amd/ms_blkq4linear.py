@@ -64,12 +64,18 @@ class BlkQ4Linear(nn.Module):
 
     def get_extra_state(self):
         return {"block_size": self.block_size, "col_wise": self.col_wise, "has_offsets": self.has_offsets,
-                "in_features": self.in_features, "out_features": self.out_features}
+                "in_features": self.in_features, "out_features": self.out_features,
+                "dtype": str(self.q_scales.dtype)}
 
     def set_extra_state(self, state):
         for key in ("block_size", "col_wise", "has_offsets", "in_features", "out_features"):
             if getattr(self, key) != state[key]:
                 raise ValueError(f"state dict was saved with {key}={state[key]}, this layer has {getattr(self, key)}")
+        # the scales of a float16 and of a bfloat16 layer are not interchangeable (copying one into the other
+        # would convert them silently); state dicts saved before the element type was recorded are float16
+        saved = state.get("dtype", "torch.float16")
+        if saved != str(self.q_scales.dtype):
+            raise ValueError(f"state dict was saved with dtype={saved}, this layer has {self.q_scales.dtype}")
 
     def forward(self, input):
         lead = input.shape[:-1]

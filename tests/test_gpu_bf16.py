@@ -327,3 +327,25 @@ def test_row_wise_gemm_on_gaussian_data(oracle, capi, device, bs, has_offsets, m
     print(f"bf16 row-wise m={m} n={n} k={k} bs={bs} zp={has_offsets}: max rel err {err:.3e}, "
           f"bit-identical outputs {float(np.mean(got == ref)):.4f}")
     assert err <= TOLERANCE
+
+
+def test_module_state_dict_round_trip_in_bfloat16(device):
+    """a bfloat16 layer's state travels like a float16 layer's, and neither takes the other's"""
+    from gemmlib_amd import ms_blkq4linear as mod
+    g = torch.Generator(device="cpu").manual_seed(12)
+    k, n, bs = 128, 64, 64
+    w = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16).to(device)
+    bias = torch.randn(n, generator=g).to(torch.bfloat16).to(device)
+    x = torch.randn(7, k, generator=g).to(torch.bfloat16).to(device)
+    layer = mod.BlkQ4Linear(bs, True, False, w, bias)
+    state = layer.state_dict()
+    other = mod.BlkQ4Linear(bs, True, False, torch.zeros_like(w), torch.zeros_like(bias))
+    other.load_state_dict(state)
+    assert other.q_scales.dtype == torch.bfloat16 and torch.equal(other(x), layer(x))
+    half = mod.BlkQ4Linear(bs, True, False, torch.zeros(n, k, dtype=torch.float16, device=device))
+    with pytest.raises((ValueError, RuntimeError)):
+        half.load_state_dict(state, strict=False)
+    with pytest.raises((ValueError, RuntimeError)):
+        other.load_state_dict(half.state_dict(), strict=False)
+    packed = mod.BlkQ4Linear.from_packed(bs, True, k, n, layer.q_weights, layer.q_scales, layer.q_zp, bias)
+    assert torch.equal(packed(x), layer(x))
