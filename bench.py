@@ -6,10 +6,14 @@
 One "step" is one call of ``blkq4_fp16_gemm_sm80`` on the headline workload (C4: the M=2048 prefill
 GEMM); the GEMV (C2) and the other configurations are measured the same way and reported inside the
 same JSON line.  Inputs are resident in HBM before the timed region.  HBM-bound configurations rotate
-over enough distinct weight sets to exceed the 256 MB Infinity Cache.  Kernel time comes from HIP
-events on the launch stream around a captured graph of back-to-back launches; wall time around the
-same region gives ``value``.  The CPU baseline is the oracle (dequantize + fp32-accumulate GEMM,
-OpenMP) on a bounded sample of the same workload, and is only a baseline.
+over distinct weight sets whose total size is at least twice the 256 MB Infinity Cache, and the timed
+graph visits every set equally often whatever ``--steps`` is.  Every configuration is replayed untimed
+until the clocks have settled.  Kernel time comes from HIP events on the launch stream around a captured
+graph of back-to-back launches (median of a few such regions); wall time around the same region gives
+``value``.  After timing, the output buffer the timed launches wrote and the packed buffers they read are
+compared with the oracle (``parity`` in the JSON line; a mismatch makes the exit code 1).  The CPU baseline
+is the oracle (quantize, dequantize + fp32-accumulate GEMM, OpenMP) on a bounded sample of the same
+workload, reported next to every GPU figure, and is only a baseline.
 """
 
 from __future__ import annotations
@@ -44,9 +48,11 @@ CONFIGS = {
     "C2b": (1, 4096, 4096, 64, False, "hbm"),
 }
 BF16 = {"C4b", "C2b"}  # through blkq4_bf16_quant_sm80 / blkq4_bf16_gemm_sm80
-# workloads whose kernels run long enough for the clocks to matter: replayed untimed for a while before the
-# timed replay (a few milliseconds after an idle gap run at ramping clocks)
-SETTLE_SECONDS = {"V128K": 0.4, "B16": 0.4, "C5_prepack": 0.4}
+# every workload is replayed untimed for this long before the timed replays (a few milliseconds after an
+# idle gap run at ramping clocks: the figure wanted is the steady state, whatever --steps is)
+SETTLE_SECONDS = 0.4
+TIMED_REGIONS = 5       # the reported time is the median over this many timed regions of the same graph
+TOLERANCE = 1e-2        # max |got - ref| / max(|ref|, 1e-3 max|ref|) against the oracle
 COLUMN_WISE = {"C4r": False, "C2r": False}
 DESCRIPTION = {
     "C1": "C1 CPU-runnable case M=64 K=1024 N=1024 bs32 asym",
@@ -106,9 +112,11 @@ def prepack_bytes(k, n, bs, has_offsets):
     return 2 * k * n + k * n // 2 + 2 * k * n // bs + (k * n // bs if has_offsets else 0)
 
 
-def timed_region(torch, launches, steps, warmup, settle_seconds=0.0):
+def timed_region(torch, launches, steps, warmup, settle_seconds=SETTLE_SECONDS, regions=TIMED_REGIONS):
     """launches: list of zero-argument callables that each enqueue ONE kernel on the current stream;
-    call i uses launches[i % len].  Returns (wall seconds, event seconds, 'graph'|'eager')."""
+    call i uses launches[i % len].  A region is `steps` back-to-back launches (one graph replay), bracketed by
+    synchronize on both sides; the median over `regions` regions is returned as
+    (wall seconds, event seconds, 'graph'|'eager')."""
     nl = len(launches)
     for i in range(warmup):
         launches[i % nl]()
@@ -127,44 +135,72 @@ def timed_region(torch, launches, steps, warmup, settle_seconds=0.0):
         torch.cuda.synchronize()
         graph.replay()  # untimed: first replay uploads the graph
         torch.cuda.synchronize()
-        t_settle = time.perf_counter()
-        while time.perf_counter() - t_settle < settle_seconds:
-            graph.replay()
-            torch.cuda.synchronize()
     except Exception as e:  # pragma: no cover - depends on the runtime
         sys.stderr.write(f"[bench] graph capture unavailable ({type(e).__name__}: {e}); timing eager launches\n")
         graph = None
         mode = "eager"
         torch.cuda.synchronize()
-    ev0 = torch.cuda.Event(enable_timing=True)
-    ev1 = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ev0.record()
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(steps):
-            launches[i % nl]()
-    ev1.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    return t1 - t0, ev0.elapsed_time(ev1) * 1e-3, mode
+
+    def region():
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                launches[i % nl]()
+
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < settle_seconds:
+        for _ in range(4):
+            region()
+        torch.cuda.synchronize()
+    walls, evts = [], []
+    for _ in range(regions):
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0.record()
+        region()
+        ev1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        walls.append(t1 - t0)
+        evts.append(ev0.elapsed_time(ev1) * 1e-3)
+    walls.sort()
+    evts.sort()
+    return walls[len(walls) // 2], evts[len(evts) // 2], mode
+
+
+def np_view(t):
+    """device or host tensor (fp16 / bf16 / uint8) -> numpy array of the same bits (fp16 as float16, bf16 as uint16)."""
+    import numpy as np
+    import torch
+    t = t.detach().cpu().contiguous()
+    if t.dtype == torch.float16:
+        return t.view(torch.int16).numpy().view(np.float16)
+    if t.dtype == torch.bfloat16:
+        return t.view(torch.int16).numpy().view(np.uint16)
+    return t.numpy()
 
 
 def make_problem(torch, capi, name, device, copies):
+    """Inputs of one workload, resident on the device.  The LAST weight set comes from the seeded CPU generator
+    (its fp16 source is kept on the host for the oracle); the sets before it are drawn on the device."""
     m, k, n, bs, has_offsets, _ = CONFIGS[name]
     col = COLUMN_WISE.get(name, True)
     bf = name in BF16
     dtype = torch.bfloat16 if bf else torch.float16
     g = torch.Generator(device="cpu").manual_seed(1234 + list(CONFIGS).index(name))
     a = torch.randn(m, k, generator=g, dtype=torch.float32).to(dtype).to(device)
+    w_host = (torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).to(dtype)
+    gd = torch.Generator(device=device).manual_seed(99 + list(CONFIGS).index(name))
     w_elems, meta_elems = capi.quant_size(bs, col, k, n)
     sets = []
-    w_host = None
     for c in range(copies):
-        w_host = (torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).to(dtype)
-        w = w_host.to(device)
+        if c == copies - 1:
+            w = w_host.to(device)
+        else:
+            w = (torch.randn(n, k, generator=gd, dtype=torch.float32, device=device) * 0.02).to(dtype)
         q_w = torch.empty(w_elems, dtype=torch.uint8, device=device)
         q_s = torch.empty(meta_elems, dtype=dtype, device=device)
         q_zp = torch.empty(meta_elems, dtype=torch.uint8, device=device) if has_offsets else None
@@ -172,17 +208,76 @@ def make_problem(torch, capi, name, device, copies):
         sets.append((q_w, q_s, q_zp))
         del w
     torch.cuda.synchronize()
-    out = torch.empty(m, n, dtype=dtype, device=device)
+    out = torch.full((m, n), float("nan"), dtype=dtype, device=device)
     return a, sets, out, w_host
 
 
-def bench_gemm(torch, capi, name, device, steps, warmup):
+def check_and_baseline(name, a_dev, last_set, out_dev, w_host, with_cpu=True):
+    """Parity gate and CPU baseline of one workload, both from the oracle on the host.
+
+    Parity: the packed weights, scales and zero-points the timed launches read (the last weight set) against the
+    oracle's quantizer, byte for byte; the output buffer the last timed launch wrote against the oracle's
+    dequantize + GEMM (every row up to 64 rows, else a spread sample of rows).
+    CPU baseline: the same oracle calls, timed: dequantize (whole B) + GEMM over a bounded number of rows."""
+    import numpy as np
+    from oracle import blkq4_oracle as O
+    m, k, n, bs, has_offsets, bound = CONFIGS[name]
+    col = COLUMN_WISE.get(name, True)
+    bf = name in BF16
+    w = np_view(w_host)
+    a = np_view(a_dev)
+    t0 = time.perf_counter()
+    canon, s, z = O.quantize(bs, col, w, has_offsets, bf16=bf)
+    t_quant = time.perf_counter() - t0
+    ps, pz = O.prepack_meta_sm80(bs, col, k, n, s.view(np.float16) if bf else s, z)
+    q_w, q_s, q_zp = last_set
+    prepack_ok = bool(np.array_equal(np_view(q_w), O.native_from_canonical(canon).reshape(-1))
+                      and np.array_equal(np_view(q_s).view(np.uint16).reshape(-1), ps.view(np.uint16).reshape(-1))
+                      and (q_zp is None or np.array_equal(np_view(q_zp).reshape(-1), pz.reshape(-1))))
+    t0 = time.perf_counter()
+    b = O.dequantize(bs, col, canon, s, z, bf16=bf)
+    t_deq = time.perf_counter() - t0
+    if m <= 64:
+        rows = np.arange(m)
+    else:
+        want = 64 if m * n * k <= (1 << 36) else 12
+        rows = np.unique(np.concatenate([np.linspace(0, m - 1, want).astype(np.int64), [0, m - 1]]))
+    a_rows = np.ascontiguousarray(a[rows])
+    t0 = time.perf_counter()
+    ref = O.gemm(a_rows, b, bf16=bf)
+    t_gemm = time.perf_counter() - t0
+    got = np_view(out_dev)[rows]
+    if bf:
+        got, ref = O.bf16_to_f32(got), O.bf16_to_f32(ref)
+    g64, r64 = got.astype(np.float64), ref.astype(np.float64)
+    floor = 1e-3 * float(np.max(np.abs(r64))) + 1e-30
+    err = float(np.max(np.abs(g64 - r64) / np.maximum(np.abs(r64), floor))) if np.all(np.isfinite(g64)) else float("inf")
+    parity = {"prepack_bit_exact": prepack_ok, "gemm_max_rel_err": float(f"{err:.3e}"), "rows_checked": int(len(rows)),
+              "of_rows": m, "ok": bool(prepack_ok and err <= TOLERANCE)}
+    base = None
+    if with_cpu:
+        flops, nbytes = algorithmic(m, k, n, bs, has_offsets)
+        # GEMM time for the whole workload, from the rows just computed (a second, larger sample for the big ones
+        # would add minutes; the oracle's GEMM time is linear in the rows)
+        t_whole = t_deq + t_gemm * m / len(rows)
+        if bound == "mfma":
+            value, unit = flops / t_whole / 1e12, "TFLOP/s"
+        else:
+            value, unit = nbytes / t_whole / 1e9, "GB/s"
+        base = {"value": float(f"{value:.4g}"), "unit": unit, "cores": O.num_threads(), "kind": "port",
+                "sample": f"oracle dequantize of the whole B {t_deq:.3f}s + GEMM of {len(rows)} of {m} rows {t_gemm:.3f}s "
+                          f"(scaled to {m} rows); oracle quantize of B {t_quant:.3f}s = "
+                          f"{prepack_bytes(k, n, bs, has_offsets) / t_quant / 1e9:.2f} GB/s"}
+    return parity, base, t_quant
+
+
+def bench_gemm(torch, capi, name, device, steps, warmup, with_cpu=True):
     m, k, n, bs, has_offsets, bound = CONFIGS[name]
     flops, nbytes = algorithmic(m, k, n, bs, has_offsets)
     copies = 1
+    per_set = nbytes - 2 * m * k - 2 * m * n
     if bound == "hbm":
-        per_set = nbytes - 2 * m * k - 2 * m * n
-        copies = INFINITY_CACHE_BYTES // per_set + 2
+        copies = 2 * INFINITY_CACHE_BYTES // per_set + 1
     a, sets, out, w_host = make_problem(torch, capi, name, device, copies)
     col = COLUMN_WISE.get(name, True)
 
@@ -191,9 +286,11 @@ def bench_gemm(torch, capi, name, device, steps, warmup):
         return lambda: capi.gemm(bs, col, m, n, k, a, q_w, q_s, q_zp, out, bf16=name in BF16)
 
     launches = [mk(s) for s in sets]
-    wall, evt, mode = timed_region(torch, launches, steps, warmup, SETTLE_SECONDS.get(name, 0.0))
-    per_call_wall = wall / steps
-    per_call_evt = evt / steps
+    # every weight set is visited equally often, and the last launch reads the last (seeded) set
+    n_launch = copies * ((max(steps, copies) + copies - 1) // copies)
+    wall, evt, mode = timed_region(torch, launches, n_launch, warmup)
+    per_call_wall = wall / n_launch
+    per_call_evt = evt / n_launch
     if bound == "mfma":
         achieved, peak, unit = flops / per_call_evt / 1e12, PEAK_MFMA_TFLOPS, "TFLOP/s"
         value = flops / per_call_wall / 1e12
@@ -203,35 +300,58 @@ def bench_gemm(torch, capi, name, device, steps, warmup):
     res = {
         "workload": DESCRIPTION[name], "value": round(value, 3), "unit": unit,
         "ms_per_step": round(per_call_wall * 1e3, 6), "kernel_us": round(per_call_evt * 1e6, 3),
-        "timing": mode, "weight_sets": copies, "flops": flops, "bytes": nbytes,
+        "timing": mode, "launches_per_region": n_launch, "weight_sets": copies,
+        "weight_footprint_bytes": copies * per_set, "flops": flops, "bytes": nbytes,
         "tflops": round(flops / per_call_evt / 1e12, 3), "gbps": round(nbytes / per_call_evt / 1e9, 3),
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
                      "frac": round(achieved / peak, 4), "traffic": traffic_bytes(name)},
     }
+    torch.cuda.synchronize()
+    parity, base, _ = check_and_baseline(name, a, sets[-1], out, w_host, with_cpu)
+    res["parity"] = parity
+    if base is not None:
+        res["cpu_baseline"] = base
     return res, (a, sets, out, w_host)
 
 
-def bench_prepack(torch, capi, device, steps, warmup):
+def bench_prepack(torch, capi, device, steps, warmup, with_cpu=True):
+    import numpy as np
     _, k, n, bs, has_offsets, _ = CONFIGS["C5"]
     nbytes = prepack_bytes(k, n, bs, has_offsets)
     g = torch.Generator(device="cpu").manual_seed(4321)
-    w = (torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).to(torch.float16).to(device)
+    w_host = (torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).to(torch.float16)
+    w = w_host.to(device)
     w_elems, meta_elems = capi.quant_size(bs, True, k, n)
-    q_w = torch.empty(w_elems, dtype=torch.uint8, device=device)
-    q_s = torch.empty(meta_elems, dtype=torch.float16, device=device)
-    q_zp = torch.empty(meta_elems, dtype=torch.uint8, device=device)
+    q_w = torch.full((w_elems,), 0xA5, dtype=torch.uint8, device=device)
+    q_s = torch.full((meta_elems,), float("nan"), dtype=torch.float16, device=device)
+    q_zp = torch.full((meta_elems,), 0xEE, dtype=torch.uint8, device=device)
     launches = [lambda: capi.quant(bs, True, w, q_w, q_s, q_zp)]
     steps = max(10, steps // 10)
-    wall, evt, mode = timed_region(torch, launches, steps, max(2, warmup // 10), SETTLE_SECONDS["C5_prepack"])
+    wall, evt, mode = timed_region(torch, launches, steps, max(2, warmup // 10))
     per = evt / steps
     ach = nbytes / per / 1e9
-    return {
+    res = {
         "workload": "C5 quantize+prepack K=8192 N=28672 bs16 asym", "value": round(nbytes / (wall / steps) / 1e9, 3),
         "unit": "GB/s", "ms_per_step": round(wall / steps * 1e3, 6), "kernel_us": round(per * 1e6, 3), "timing": mode,
-        "bytes": nbytes, "gbps": round(ach, 3),
+        "launches_per_region": steps, "bytes": nbytes, "gbps": round(ach, 3),
         "roofline": {"bound": "hbm", "achieved": round(ach, 3), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                      "frac": round(ach / PEAK_HBM_GBPS, 4), "traffic": traffic_bytes("C5_prepack")},
     }
+    # parity: every byte the timed launches wrote, against the oracle's quantizer (timed: the CPU baseline)
+    from oracle import blkq4_oracle as O
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    canon, s, z = O.quantize(bs, True, np_view(w_host), has_offsets)
+    t_quant = time.perf_counter() - t0
+    ps, pz = O.prepack_meta_sm80(bs, True, k, n, s, z)
+    ok = bool(np.array_equal(np_view(q_w), O.native_from_canonical(canon).reshape(-1))
+              and np.array_equal(np_view(q_s).view(np.uint16), ps.view(np.uint16).reshape(-1))
+              and np.array_equal(np_view(q_zp), pz.reshape(-1)))
+    res["parity"] = {"prepack_bit_exact": ok, "bytes_checked": int(q_w.numel() + 2 * q_s.numel() + q_zp.numel()), "ok": ok}
+    if with_cpu:
+        res["cpu_baseline"] = {"value": float(f"{nbytes / t_quant / 1e9:.4g}"), "unit": "GB/s", "cores": O.num_threads(),
+                               "kind": "port", "sample": f"oracle quantize of the whole B (one run) {t_quant:.3f}s"}
+    return res
 
 
 def bench_copy(torch, capi, device, steps, warmup):
@@ -246,7 +366,7 @@ def bench_copy(torch, capi, device, steps, warmup):
     steps = max(10, steps // 10)
     for _ in range(steps):  # the runtime's own device-to-device copy of the same buffer, as a second reference
         dst.copy_(src)
-    wall, evt, mode = timed_region(torch, launches, steps, max(2, warmup // 10), SETTLE_SECONDS["C5_prepack"])
+    wall, evt, mode = timed_region(torch, launches, steps, max(2, warmup // 10))
     per = evt / steps
     ach = 2 * nbytes / per / 1e9
     return {
@@ -268,13 +388,14 @@ def bench_context(torch, capi, device, head_problem, steps, warmup):
     * a kernel that does nothing but back-to-back fp16 MFMAs (one wave per SIMD, all 256 compute units) on
       random and on all-zero operands: the rate the chip sustains, which is the ceiling of any fp16 GEMM."""
     import ctypes
-    from gemmlib_amd import build as _build
+    import bench_probe
     out = {}
-    probe = ctypes.CDLL(_build.PROBE_PATH)
+    probe = ctypes.CDLL(bench_probe.build())
     probe.blkq4_probe_empty.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
     probe.blkq4_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                          ctypes.c_void_p, ctypes.c_void_p]
     scratch = torch.zeros(1 << 16, dtype=torch.int32, device=device)
+    steps = max(steps, 100)  # the floors are small numbers: at least 100 launches per region
     probe.blkq4_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
 
     def stream_ptr():
@@ -287,19 +408,20 @@ def bench_context(torch, capi, device, head_problem, steps, warmup):
         n_launch = 20
         wall, evt, _ = timed_region(
             torch, [lambda: probe.blkq4_probe_mfma(random_operands, mfma_iters, scratch.data_ptr(), stream_ptr())],
-            n_launch, 3)
+            n_launch, 3, settle_seconds=0.2, regions=3)
         out[key] = round(256 * 4 * mfma_iters * 8 * 32768.0 / (evt / n_launch) / 1e12, 1)
     m, k, n, bs, has_offsets, _ = CONFIGS["C2"]
     per_set = k * n // 2 + 2 * k * n // bs
-    copies = INFINITY_CACHE_BYTES // per_set + 2
+    copies = 2 * INFINITY_CACHE_BYTES // per_set + 1
+    floor_launches = copies * ((max(steps, copies) + copies - 1) // copies)
     ws = [torch.randint(0, 256, (k * n // 2,), dtype=torch.uint8, device=device) for _ in range(copies)]
     ss = [torch.ones(k // bs * n, dtype=torch.float16, device=device) for _ in range(copies)]
     for with_scales in (False, True):
         launches = [(lambda w=w, sc=sc: probe.blkq4_probe_stream(w.data_ptr(), sc.data_ptr() if with_scales else None,
                                                                  n, k, scratch.data_ptr(), stream_ptr()))
                     for w, sc in zip(ws, ss)]
-        wall, evt, _ = timed_region(torch, launches, steps, warmup)
-        out["c2_requests_only_us" if with_scales else "c2_weight_requests_only_us"] = round(evt / steps * 1e6, 3)
+        wall, evt, _ = timed_region(torch, launches, floor_launches, warmup)
+        out["c2_requests_only_us" if with_scales else "c2_weight_requests_only_us"] = round(evt / floor_launches * 1e6, 3)
     del ws, ss
     if head_problem is not None:
         a, sets, c, w_host = head_problem
@@ -321,37 +443,6 @@ def bench_context(torch, capi, device, head_problem, steps, warmup):
         wall, evt, _ = timed_region(torch, [lambda: capi.gemm(bs, True, m, n, k, za, zw, zs, zz, c)], steps, warmup)
         out["c4_all_zero_data_us"] = round(evt / steps * 1e6, 3)
     return out
-
-
-def cpu_baseline(name, a_dev, w_host, target_seconds=12.0):
-    """The oracle's dequantize + GEMM on a bounded sample of rows of the same workload."""
-    import numpy as np
-    from oracle import blkq4_oracle as O
-    m, k, n, bs, has_offsets, _ = CONFIGS[name]
-    w = w_host.view(__import__("torch").int16).numpy().view(np.float16)
-    a = a_dev.cpu().view(__import__("torch").int16).numpy().view(np.float16)
-    t0 = time.perf_counter()
-    canon, s, z = O.quantize(bs, True, w, has_offsets)
-    t_quant = time.perf_counter() - t0
-    t0 = time.perf_counter()
-    b = O.dequantize(bs, True, canon, s, z)
-    t_deq = time.perf_counter() - t0
-    rows = min(m, 16)
-    t0 = time.perf_counter()
-    O.gemm(np.ascontiguousarray(a[:rows]), b)
-    t_probe = time.perf_counter() - t0
-    rows = int(max(rows, min(m, rows * target_seconds / max(t_probe, 1e-3))))
-    t0 = time.perf_counter()
-    O.gemm(np.ascontiguousarray(a[:rows]), b)
-    t_gemm = time.perf_counter() - t0
-    flops = 2.0 * rows * n * k
-    return {
-        "value": round(flops / (t_gemm + t_deq * rows / m) / 1e12, 5), "unit": "TFLOP/s",
-        "cores": O.num_threads(), "kind": "port",
-        "sample": f"{rows} of {m} rows of {DESCRIPTION[name]}: dequantize {t_deq:.3f}s (whole B, charged pro rata), "
-                  f"GEMM {t_gemm:.3f}s; oracle quantize of B {t_quant:.3f}s "
-                  f"({prepack_bytes(k, n, bs, has_offsets) / t_quant / 1e9:.2f} GB/s)",
-    }
 
 
 def main(argv=None) -> int:
@@ -377,16 +468,19 @@ def main(argv=None) -> int:
     torch.cuda.set_device(device)
 
     wanted = [c.strip() for c in args.configs.split(",") if c.strip()]
+    with_cpu = not args.no_cpu
     results = {}
     head = None
     head_problem = None
     for name in wanted:
+        sys.stderr.write(f"[bench] {name}\n")
+        sys.stderr.flush()
         if name == "prepack":
-            results["C5_prepack"] = bench_prepack(torch, capi, device, args.steps, args.warmup)
+            results["C5_prepack"] = bench_prepack(torch, capi, device, args.steps, args.warmup, with_cpu)
         elif name == "copy":
             results["copy"] = bench_copy(torch, capi, device, args.steps, args.warmup)
         else:
-            res, problem = bench_gemm(torch, capi, name, device, args.steps, args.warmup)
+            res, problem = bench_gemm(torch, capi, name, device, args.steps, args.warmup, with_cpu)
             results[name] = res
             if name == "C4":
                 head, head_problem = res, problem
@@ -396,23 +490,38 @@ def main(argv=None) -> int:
     if head is None:  # headline not requested: report the first one measured
         head = next(iter(results.values()))
 
+    checked = {k: v["parity"] for k, v in results.items() if "parity" in v}
+    parity_ok = all(v["ok"] for v in checked.values())
     line = {
         "metric": METRIC, "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": head["workload"], "timing": head.get("timing")},
+        "config": {"workload": head["workload"], "timing": head.get("timing"),
+                   "launches_per_timed_region": head.get("launches_per_region"), "timed_regions": TIMED_REGIONS,
+                   "settle_seconds": SETTLE_SECONDS},
         "roofline": head["roofline"],
+        "parity": {"ok": parity_ok, "tolerance": TOLERANCE,
+                   "metric": "max |got - ref| / max(|ref|, 1e-3 max|ref|) against the oracle; prepack byte for byte",
+                   "checked": checked},
     }
+    if "cpu_baseline" in head:
+        line["cpu_baseline"] = head["cpu_baseline"]
     if "C2" in results:
-        line["gemv"] = {"workload": results["C2"]["workload"], "value": results["C2"]["value"], "unit": "GB/s",
-                        "kernel_us": results["C2"]["kernel_us"], "roofline": results["C2"]["roofline"]}
+        c2 = results["C2"]
+        line["gemv"] = {"workload": c2["workload"], "value": c2["value"], "unit": "GB/s",
+                        "kernel_us": c2["kernel_us"], "roofline": c2["roofline"], "weight_sets": c2["weight_sets"],
+                        "weight_footprint_bytes": c2["weight_footprint_bytes"],
+                        "launches_per_timed_region": c2["launches_per_region"]}
+        if "cpu_baseline" in c2:
+            line["gemv"]["cpu_baseline"] = c2["cpu_baseline"]
     if not args.no_context:
+        sys.stderr.write("[bench] context\n")
         line["context"] = bench_context(torch, capi, device, head_problem, args.steps, args.warmup)
-    if not args.no_cpu and head_problem is not None:
-        a, sets, out, w_host = head_problem
-        line["cpu_baseline"] = cpu_baseline("C4", a, w_host)
     line["all"] = results
     print(json.dumps(line))
+    if not parity_ok:
+        sys.stderr.write("[bench] PARITY FAILED: " + json.dumps({k: v for k, v in checked.items() if not v["ok"]}) + "\n")
+        return 1
     return 0
 
 

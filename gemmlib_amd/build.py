@@ -1,7 +1,9 @@
 """Builds the native parts in-tree:
 
 * ``gemmlib_amd/lib/libms_blkq4gemm.so`` -- the C-ABI library (host code + gfx950 HIP kernels);
-* ``gemmlib_amd/ms_blkq4linear_ext*.so`` -- the PyTorch-ROCm extension on top of it (optional).
+* ``ms_blkq4linear_ext*.so`` at the top of the tree, next to ``ms_blkq4linear.py`` -- the PyTorch-ROCm
+  extension on top of it, importable as the reference's is: ``import ms_blkq4linear_ext``
+  (reference: python/ms_blkq4linear.py:7, python/setup.py:17-26).
 
 Run as ``python -m gemmlib_amd.build [--no-ext]``.  hipcc cross-compiles for gfx950, so no GPU is
 needed to build.
@@ -23,7 +25,6 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 OBJ_DIR = os.path.join(PKG_DIR, "build")
 INCLUDE = os.path.join(ROOT, "include")
 LIB_PATH = os.path.join(LIB_DIR, "libms_blkq4gemm.so")
-PROBE_PATH = os.path.join(LIB_DIR, "libblkq4_probe.so")  # measurement aids for bench.py, not part of the product
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -71,7 +72,6 @@ def build_library(verbose: bool = True) -> str:
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
         list(pool.map(lambda j: _run(*j), jobs))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs], "packed-fp32-ops")
-    _run([HIPCC, *HIP_FLAGS, "-shared", "-o", PROBE_PATH, os.path.join(CSRC, "blkq4_probe.hip")], "packed-fp32-ops")
     if verbose:
         print(f"built {LIB_PATH}")
     return LIB_PATH
@@ -79,16 +79,17 @@ def build_library(verbose: bool = True) -> str:
 
 def ext_path() -> str:
     suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
-    return os.path.join(PKG_DIR, "ms_blkq4linear_ext" + suffix)
+    return os.path.join(ROOT, "ms_blkq4linear_ext" + suffix)
 
 
-def build_extension(verbose: bool = True) -> str:
+def build_extension(verbose: bool = True, out: str | None = None) -> str:
     """The pybind11/torch extension, compiled as plain C++ against PyTorch-ROCm and linked to the
-    C-ABI library (no hipify pass, no CUDA headers)."""
+    C-ABI library (no hipify pass, no CUDA headers).  It finds the library at ``gemmlib_amd/lib`` next to
+    itself, in the source tree and in an installed one alike."""
     import torch
     from torch.utils import cpp_extension
 
-    out = ext_path()
+    out = out or ext_path()
     torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
     inc = []
     for p in cpp_extension.include_paths():
@@ -101,7 +102,7 @@ def build_extension(verbose: bool = True) -> str:
         "-Wno-deprecated-declarations",
         *inc, "-I", INCLUDE,
         os.path.join(CSRC, "ms_blkq4linear_ext.cpp"), "-o", out,
-        "-L", LIB_DIR, "-lms_blkq4gemm", "-Wl,-rpath,$ORIGIN/lib",
+        "-L", LIB_DIR, "-lms_blkq4gemm", "-Wl,-rpath,$ORIGIN/gemmlib_amd/lib",
         "-L", torch_lib, "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip", "-ltorch_python",
         "-Wl,-rpath," + torch_lib,
     ]

@@ -79,11 +79,13 @@ int quant_size(int block_size, bool column_wise, int rows, int columns, int64_t&
   const int meta_cols = columns / kcol;
   // The reference divides by the meta extent (which is zero when the matrix is smaller than one
   // block, a division by zero there); such shapes are reported as not quantizable here.
-  if (rows < 0 || (rows % 64) != 0 || meta_rows == 0 || (rows % meta_rows) != 0) {
+  // (rows % krow, columns % kcol: a matrix that is no whole number of blocks; the reference's `% meta extent`
+  // lets some of those through, e.g. 96 columns in blocks of 64, and its kernels then write out of bounds)
+  if (rows < 0 || (rows % 64) != 0 || meta_rows == 0 || (rows % meta_rows) != 0 || (rows % krow) != 0) {
     set_error(err, "Cannot block quantize matrix with rows: " + std::to_string(rows));
     return -1;
   }
-  if (columns < 0 || (columns % 32) != 0 || meta_cols == 0 || (columns % meta_cols) != 0) {
+  if (columns < 0 || (columns % 32) != 0 || meta_cols == 0 || (columns % meta_cols) != 0 || (columns % kcol) != 0) {
     set_error(err, "Cannot block quantize matrix with columns: " + std::to_string(columns));
     return -1;
   }
@@ -289,7 +291,10 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
     set_error(err, "Kernel execution failed: Error Invalid Problem");
     return -1;
   }
-  if ((reinterpret_cast<uintptr_t>(scales_ptr) & 1u) != 0 || !aligned16(output_ptr) || (n % 8) != 0) {
+  // scales and zero-points: 4-byte aligned for every m (the tile kernel copies them four bytes at a time, and
+  // which kernel runs depends on m: one rule for all of them)
+  if ((reinterpret_cast<uintptr_t>(scales_ptr) & 3u) != 0 ||
+      (has_offsets && (reinterpret_cast<uintptr_t>(offsets_ptr) & 3u) != 0) || !aligned16(output_ptr) || (n % 8) != 0) {
     set_error(err, "Kernel execution failed: Error Misaligned Operand");
     return -1;
   }

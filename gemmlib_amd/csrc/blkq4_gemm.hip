@@ -48,6 +48,7 @@
 
 #include "blkq4_dequant.h"
 #include "blkq4_device.h"
+#include "blkq4_launch.h"
 #include "blkq4_gemm_common.h"
 
 // This file is compiled twice: as it is for fp16, and through blkq4_gemm_bf16.hip, which defines BLKQ4_GEMM_BF16
@@ -595,12 +596,13 @@ int launch_one(const blkq4_gemm_args* a) {
   const int m_tiles = (a->m + BM - 1) / BM;
   const int n_tiles = (a->n + kBN - 1) / kBN;
   const dim3 grid(static_cast<unsigned>(m_tiles) * n_tiles);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW, ROW>), grid, dim3(64 * (WM * WN + PW)), 0,
-                     static_cast<hipStream_t>(a->stream), static_cast<const uint8_t*>(a->a),
-                     static_cast<const uint8_t*>(a->packed_w), static_cast<const uint8_t*>(a->scales),
-                     static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c),
-                     static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k, m_tiles);
-  return static_cast<int>(hipGetLastError());
+  // the launch's own status: a sticky error of an earlier, unrelated call stays where it is
+  return static_cast<int>(launch_status(gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW, ROW>, grid,
+                                        dim3(64 * (WM * WN + PW)), 0, a->stream, static_cast<const uint8_t*>(a->a),
+                                        static_cast<const uint8_t*>(a->packed_w),
+                                        static_cast<const uint8_t*>(a->scales),
+                                        static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c),
+                                        static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k, m_tiles));
 }
 
 template <int BS, bool HAS_ZP>
@@ -630,14 +632,10 @@ int launch_rt(const blkq4_gemm_args* a) {
   if (a->m <= 32) return launch_one<BS, HAS_ZP, 1, 1, 1, 8, 0>(a);
   if (a->m <= 64 && one_round_of_128) return launch_one<BS, HAS_ZP, 2, 1, 1, 4, 4>(a);
   if (a->m <= 64) return launch_one<BS, HAS_ZP, 2, 1, 1, 8, 0>(a);
-#ifdef BLKQ4_GEMM_SHAPE
-  return launch_one<BS, HAS_ZP, BLKQ4_GEMM_SHAPE>(a);
-#else
   if (tiles >= kComputeUnits) return launch_one<BS, HAS_ZP, 8, 2, 1, 4, 0>(a);
   if (smallest_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 2, 1, 1, 4, 4>(a);
   if (small_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 4, 1, 1, 4, 4>(a);
   return launch_one<BS, HAS_ZP, 4, 2, 1, 4, 4>(a);
-#endif
 }
 
 template <int BS>

@@ -11,18 +11,23 @@ namespace blkq4 {
 // Asynchronous copy: every active lane moves 16 (4) bytes from global memory to
 // LDS[lds_base + lane * 16 (4)].  lds_base and base are wave-uniform, offset is per lane.  The
 // compiler does not see the LDS write; it is ordered by hand with wait_vmcnt + s_barrier.
+// M0 is named as clobbered so that the compiler never carries a value of its own in it across these
+// statements (it warns that M0 is a reserved register; the clobber is recorded all the same).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void async_copy_16(uint32_t lds_base, const void* base, uint32_t offset) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(offset), "s"(base)
-               : "memory");
+               : "memory", "m0");
 }
 // the same with the non-temporal hint, for data that this launch reads once
 __device__ __forceinline__ void async_copy_16_once(uint32_t lds_base, const void* base, uint32_t offset) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_base), "v"(offset), "s"(base)
-               : "memory");
+               : "memory", "m0");
 }
 __device__ __forceinline__ void async_copy_4_flat(uint32_t lds_base, const void* gptr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_base), "v"(gptr) : "memory", "m0");
 }
+#pragma clang diagnostic pop
 // LDS reads at byte address `addr` + `imm`.  `imm` is a compile-time constant applied as a pointer offset,
 // which the compiler folds into the instruction's offset field (it will not do that for an integer addition,
 // which may wrap); `addr` costs whatever the caller spends on it and nothing more.

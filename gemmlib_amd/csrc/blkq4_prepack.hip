@@ -18,6 +18,7 @@
 #include <stdint.h>
 
 #include "blkq4_device.h"
+#include "blkq4_launch.h"
 
 namespace {
 
@@ -436,74 +437,33 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__
   }
 }
 
-template <int BS>
-int launch_prepack_rowwise(const blkq4_prepack_args* a) {
-  const unsigned k_tiles = (a->rows + kTileK - 1) / kTileK;
-  const dim3 grid(k_tiles * static_cast<unsigned>((a->columns + kTileN - 1) / kTileN));
-  const dim3 block(kThreads);
-  hipStream_t stream = static_cast<hipStream_t>(a->stream);
-  const auto* src = static_cast<const uint16_t*>(a->src);
-  auto* pw = static_cast<uint4*>(a->packed_w);
-  auto* sc = static_cast<uint16_t*>(a->scales);
-  auto* zp = static_cast<uint8_t*>(a->zero_points);
-  const bool aligned = (reinterpret_cast<uintptr_t>(a->src) & 15u) == 0 && (a->ld % 8) == 0;
-#define BLKQ4_LAUNCH(ZP_, AL_, BF_)                                                                                   \
-  hipLaunchKernelGGL((prepack_rowwise_kernel<BS, ZP_, AL_, BF_>), grid, block, 0, stream, src, a->rows, a->columns, \
-                     a->ld, pw, sc, zp, k_tiles)
-  if (a->bf16) {
-    if (zp) {
-      if (aligned) BLKQ4_LAUNCH(true, true, true); else BLKQ4_LAUNCH(true, false, true);
-    } else {
-      if (aligned) BLKQ4_LAUNCH(false, true, true); else BLKQ4_LAUNCH(false, false, true);
-    }
-  } else if (zp) {
-    if (aligned) BLKQ4_LAUNCH(true, true, false); else BLKQ4_LAUNCH(true, false, false);
-  } else {
-    if (aligned) BLKQ4_LAUNCH(false, true, false); else BLKQ4_LAUNCH(false, false, false);
-  }
-#undef BLKQ4_LAUNCH
-  return static_cast<int>(hipGetLastError());
-}
-
+// All instantiations of a prepack kernel share one signature; `launch` starts the chosen one and returns the
+// launch's own status.
 template <int BS>
 int launch_prepack(const blkq4_prepack_args* a) {
-  if (!a->column_wise) return launch_prepack_rowwise<BS>(a);
   const unsigned k_tiles = (a->rows + kTileK - 1) / kTileK;
   const dim3 grid(k_tiles * static_cast<unsigned>((a->columns + kTileN - 1) / kTileN));
-  const dim3 block(kThreads);
-  hipStream_t stream = static_cast<hipStream_t>(a->stream);
-  const auto* src = static_cast<const uint16_t*>(a->src);
-  auto* pw = static_cast<uint4*>(a->packed_w);
-  auto* sc = static_cast<uint16_t*>(a->scales);
-  auto* zp = static_cast<uint8_t*>(a->zero_points);
   const bool aligned = (reinterpret_cast<uintptr_t>(a->src) & 15u) == 0 && (a->ld % 8) == 0;
-  const bool has_zp = zp != nullptr;
-  if (a->bf16) {
-#define BLKQ4_LAUNCH(ZP_, AL_)                                                                                     \
-  hipLaunchKernelGGL((prepack_kernel<BS, ZP_, AL_, true>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, \
-                     pw, sc, zp, k_tiles)
-    if (has_zp) {
-      if (aligned) BLKQ4_LAUNCH(true, true); else BLKQ4_LAUNCH(true, false);
-    } else {
-      if (aligned) BLKQ4_LAUNCH(false, true); else BLKQ4_LAUNCH(false, false);
-    }
-#undef BLKQ4_LAUNCH
-    return static_cast<int>(hipGetLastError());
+  const bool has_zp = a->zero_points != nullptr;
+  auto launch = [&](auto* kernel) {
+    return static_cast<int>(blkq4::launch_status(kernel, grid, dim3(kThreads), 0, a->stream,
+                                          static_cast<const uint16_t*>(a->src), a->rows, a->columns, a->ld,
+                                          static_cast<uint4*>(a->packed_w), static_cast<uint16_t*>(a->scales),
+                                          static_cast<uint8_t*>(a->zero_points), k_tiles));
+  };
+  // (has zero-points, aligned source, bf16) -> instantiation
+#define BLKQ4_PICK(KERNEL_)                                                                   \
+  if (a->bf16) {                                                                              \
+    if (has_zp) return aligned ? launch(KERNEL_<BS, true, true, true>) : launch(KERNEL_<BS, true, false, true>);   \
+    return aligned ? launch(KERNEL_<BS, false, true, true>) : launch(KERNEL_<BS, false, false, true>);             \
+  }                                                                                           \
+  if (has_zp) return aligned ? launch(KERNEL_<BS, true, true, false>) : launch(KERNEL_<BS, true, false, false>);   \
+  return aligned ? launch(KERNEL_<BS, false, true, false>) : launch(KERNEL_<BS, false, false, false>);
+  if (!a->column_wise) {
+    BLKQ4_PICK(prepack_rowwise_kernel)
   }
-  if (has_zp) {
-    if (aligned) {
-      hipLaunchKernelGGL((prepack_kernel<BS, true, true>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, pw, sc, zp, k_tiles);
-    } else {
-      hipLaunchKernelGGL((prepack_kernel<BS, true, false>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, pw, sc, zp, k_tiles);
-    }
-  } else {
-    if (aligned) {
-      hipLaunchKernelGGL((prepack_kernel<BS, false, true>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, pw, sc, zp, k_tiles);
-    } else {
-      hipLaunchKernelGGL((prepack_kernel<BS, false, false>), grid, block, 0, stream, src, a->rows, a->columns, a->ld, pw, sc, zp, k_tiles);
-    }
-  }
-  return static_cast<int>(hipGetLastError());
+  BLKQ4_PICK(prepack_kernel)
+#undef BLKQ4_PICK
 }
 
 }  // namespace
@@ -525,15 +485,10 @@ extern "C" int blkq4_dev_prepack(const blkq4_prepack_args* a) {
 extern "C" int blkq4_dev_repack(const blkq4_repack_args* a) {
   const size_t units = static_cast<size_t>(a->rows / 32) * a->columns;
   const dim3 grid(static_cast<unsigned>((units + 255) / 256));
-  hipStream_t stream = static_cast<hipStream_t>(a->stream);
   const auto* src = static_cast<const uint8_t*>(a->src);
   auto* dst = static_cast<uint8_t*>(a->dst);
-  if (a->to_sm80) {
-    hipLaunchKernelGGL((repack_kernel<true>), grid, dim3(256), 0, stream, src, dst, a->rows, a->columns);
-  } else {
-    hipLaunchKernelGGL((repack_kernel<false>), grid, dim3(256), 0, stream, src, dst, a->rows, a->columns);
-  }
-  return static_cast<int>(hipGetLastError());
+  auto* kernel = a->to_sm80 ? repack_kernel<true> : repack_kernel<false>;
+  return static_cast<int>(blkq4::launch_status(kernel, grid, dim3(256), 0, a->stream, src, dst, a->rows, a->columns));
 }
 
 extern "C" const char* blkq4_dev_error_string(int code) {

@@ -35,10 +35,9 @@
 
 #include <stdint.h>
 
-#include <atomic>
-
 #include "blkq4_dequant.h"
 #include "blkq4_device.h"
+#include "blkq4_launch.h"
 #include "blkq4_gemm_common.h"
 
 // This file is compiled twice: as it is for fp16, and through blkq4_skinny_bf16.hip, which defines
@@ -53,15 +52,11 @@ namespace {
 
 using namespace blkq4;
 
-// the packed weights are read once per launch
-#ifdef BLKQ4_W_TEMPORAL
-__device__ __forceinline__ uint4 BLKQ4_W_LOAD(const uint4_t* p) { const uint4_t v = *p; return make_uint4(v[0], v[1], v[2], v[3]); }
-#else
+// the packed weights are read once per launch: non-temporal
 __device__ __forceinline__ uint4 BLKQ4_W_LOAD(const uint4_t* p) {
   const uint4_t v = __builtin_nontemporal_load(p);
   return make_uint4(v[0], v[1], v[2], v[3]);
 }
-#endif
 
 #ifdef BLKQ4_SKINNY_BF16
 constexpr bool kBF = true;
@@ -500,18 +495,10 @@ void choose_shape(int m, int n, int k, int* nt, int* depth) {
   *depth = (*nt == 1 && tiles <= 2 * kComputeUnits) ? 8 : 4;
 }
 
-// Raises a kernel's dynamic-LDS limit, once per kernel and device (the attribute belongs to the device's copy
-// of the code).
-template <class Kernel>
-hipError_t raise_lds_limit(Kernel* kernel) {
-  static std::atomic<uint64_t> done{0};  // one flag per device index below 64, one set of flags per kernel
-  int device = 0;
-  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
-  if (device < 64 && ((done.load(std::memory_order_acquire) >> device) & 1u) != 0) return hipSuccess;
-  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
-  if (e == hipSuccess && device < 64) done.fetch_or(uint64_t{1} << device, std::memory_order_release);
-  return e;
+// Raises a kernel's dynamic-LDS limit, once per kernel instantiation and device.
+template <auto kKernel>
+hipError_t raise_lds_limit() {
+  return raise_lds_limit_once(reinterpret_cast<const void*>(kKernel), kMaxLdsBytes, &lds_limit_flags<kKernel>());
 }
 
 // One kernel instantiation: raises its dynamic-LDS limit, then launches `row_groups` row groups of
@@ -554,23 +541,23 @@ int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
   const bool refill = cg_stride < col_groups || kSplit == 1;
   auto launch = [&](auto* kernel, hipError_t attr) {
     if (attr != hipSuccess) return static_cast<int>(attr);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * kWaves), lds_bytes, static_cast<hipStream_t>(a->stream),
-                       static_cast<const uint16_t*>(a->a), static_cast<const uint4*>(a->packed_w),
-                       static_cast<const uint16_t*>(a->scales), static_cast<const uint8_t*>(a->zero_points),
-                       static_cast<uint16_t*>(a->c), static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k,
-                       rows_log2, row_groups, cg_stride,
-                       static_cast<uint32_t>(red_offset));
-    return static_cast<int>(hipGetLastError());
+    // the launch's own status: a sticky error of an earlier, unrelated call stays where it is
+    return static_cast<int>(launch_status(kernel, dim3(grid), dim3(64 * kWaves), lds_bytes, a->stream,
+                                          static_cast<const uint16_t*>(a->a), static_cast<const uint4*>(a->packed_w),
+                                          static_cast<const uint16_t*>(a->scales),
+                                          static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c),
+                                          static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k, rows_log2,
+                                          row_groups, cg_stride, static_cast<uint32_t>(red_offset)));
   };
   if (refill) {
-    auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, true, kSplit>;
-    return launch(kernel, raise_lds_limit(kernel));
+    constexpr auto kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, true, kSplit>;
+    return launch(kernel, raise_lds_limit<kernel>());
   }
   if constexpr (kSplit == 1) {
     return static_cast<int>(hipErrorInvalidValue);  // not reached
   } else {
-    auto* kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, false, kSplit>;
-    return launch(kernel, raise_lds_limit(kernel));
+    constexpr auto kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, false, kSplit>;
+    return launch(kernel, raise_lds_limit<kernel>());
   }
 }
 

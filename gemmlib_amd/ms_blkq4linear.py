@@ -21,7 +21,7 @@ them, and takes 2-D inputs only):
 import torch
 from torch import nn
 
-from . import ms_blkq4linear_ext
+import ms_blkq4linear_ext  # top-level, as in the reference (python/ms_blkq4linear.py:7)
 
 
 class BlkQ4Linear(nn.Module):

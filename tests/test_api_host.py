@@ -59,6 +59,9 @@ def test_quant_size_closed_form(capi, oracle, bs, col, rows, cols, w, meta):
     ((64, True, 32, 32), "Cannot block quantize matrix with rows: 32"),
     ((32, True, 64, 48), "Cannot block quantize matrix with columns: 48"),
     ((64, False, 64, 32), "Cannot block quantize matrix with columns: 32"),  # fewer columns than one block
+    # a multiple of 32 that is no whole number of blocks (the reference's `columns % meta columns` lets it through)
+    ((64, False, 64, 96), "Cannot block quantize matrix with columns: 96"),
+    ((64, False, 128, 160), "Cannot block quantize matrix with columns: 160"),
 ])
 def test_quant_size_errors(capi, args, message):
     with pytest.raises(capi.Blkq4Error) as e:
@@ -99,6 +102,10 @@ def _gemm(capi, bs=32, col=True, m=4, n=64, k=64, a=None, w=None, s=None, z=None
      "Kernel execution failed: Error Invalid Problem"),
     (dict(a=_buf(512, address=0x1002)), "Kernel execution failed: Error Misaligned Operand"),
     (dict(c=_buf(512, address=0x1008)), "Kernel execution failed: Error Misaligned Operand"),
+    # scales and zero-points are copied four bytes at a time by the tile kernel: one rule for every m
+    (dict(s=_buf(256, address=0x1002)), "Kernel execution failed: Error Misaligned Operand"),
+    (dict(z=_buf(128, address=0x1001)), "Kernel execution failed: Error Misaligned Operand"),
+    (dict(m=2048, z=_buf(128, address=0x1002)), "Kernel execution failed: Error Misaligned Operand"),
     # the entry point with a bias: its size and alignment, and the checks of the plain one in the same order
     (dict(bias=_buf(126)), "Unexpected bias tensor size: 126 expected: 128"),
     (dict(bias=_buf(128, address=0x1008)), "Kernel execution failed: Error Misaligned Operand"),

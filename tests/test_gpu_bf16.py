@@ -228,7 +228,7 @@ def test_packed_weights_and_offsets_are_those_of_the_fp16_quantizer(oracle, capi
 def test_module_takes_bfloat16(oracle, capi, device, scale_only, m):
     """BlkQ4Linear built from bfloat16 weights: bfloat16 scales, bias and output, the result that of the C entry
     points (which the tests above hold against the oracle); a float16 input to such a layer is refused"""
-    from gemmlib_amd import ms_blkq4linear as mod
+    import ms_blkq4linear as mod
     g = torch.Generator(device="cpu").manual_seed(13 + m)
     k, n, bs = 512, 384, 64
     w = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16)
@@ -331,7 +331,7 @@ def test_row_wise_gemm_on_gaussian_data(oracle, capi, device, bs, has_offsets, m
 
 def test_module_state_dict_round_trip_in_bfloat16(device):
     """a bfloat16 layer's state travels like a float16 layer's, and neither takes the other's"""
-    from gemmlib_amd import ms_blkq4linear as mod
+    import ms_blkq4linear as mod
     g = torch.Generator(device="cpu").manual_seed(12)
     k, n, bs = 128, 64, 64
     w = (torch.randn(n, k, generator=g) * 0.02).to(torch.bfloat16).to(device)

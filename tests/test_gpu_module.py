@@ -13,13 +13,13 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(scope="module")
 def mod():
-    from gemmlib_amd import ms_blkq4linear  # fails loudly if the extension is not built
+    import ms_blkq4linear  # top-level, as a user of the reference imports it; fails loudly if the extension is not built
     return ms_blkq4linear
 
 
 def test_quant_matches_known_answer(oracle, device, mod):
     """the reference script's construction: in=64, out=32, block 32 (here column-wise)."""
-    from gemmlib_amd import ms_blkq4linear_ext as ext
+    import ms_blkq4linear_ext as ext
     kat = oracle.kat_generate(32, True, 64, 32, True)
     q_w, q_s, q_zp = ext.quant(32, True, True, to_dev(kat["weights"], device))
     assert q_w.dtype == torch.uint8 and q_w.dim() == 1 and q_w.numel() == 64 * 32 // 2
@@ -51,7 +51,7 @@ def test_module_forward_with_bias(oracle, device, mod, scale_only, m):
 
 
 def test_extension_argument_checks(device, mod):
-    from gemmlib_amd import ms_blkq4linear_ext as ext
+    import ms_blkq4linear_ext as ext
     w = torch.zeros(32, 64, dtype=torch.float16, device=device)
     with pytest.raises(RuntimeError, match="only supports float16 weights"):
         ext.quant(32, True, True, w.float())
@@ -109,3 +109,28 @@ def test_state_dict_round_trip_and_from_packed(device, mod):
     assert torch.equal(packed(x), layer(x))
     with pytest.raises(ValueError):
         mod.BlkQ4Linear.from_packed(bs, True, k, n + 32, layer.q_weights, layer.q_scales, layer.q_zp)
+
+
+def test_reference_usage_script_steps_with_plain_imports_then_forward(oracle, device):
+    """What a user of the reference runs (reference: python/blkq4linear_test.py:5-85): plain ``import
+    ms_blkq4linear``, in_features 64, out_features 32, blocks of 32 along out_features, weights built from the
+    known-answer quantized data, ``BlkQ4Linear(block_size, col_wise, scale_only, weights)``; then the packed
+    tensors are what the construction started from, and ``forward`` (which that script never calls) is exact."""
+    import importlib
+    ms_blkq4linear = importlib.import_module("ms_blkq4linear")
+    ext = importlib.import_module("ms_blkq4linear_ext")
+    assert "gemmlib_amd" not in ms_blkq4linear.__name__ and ext.__name__ == "ms_blkq4linear_ext"
+    in_features, out_features, block_size, col_wise, scale_only = 64, 32, 32, False, False
+    kat = oracle.kat_generate(block_size, col_wise, in_features, out_features, not scale_only)
+    weights = to_dev(kat["weights"], device)
+    layer = ms_blkq4linear.BlkQ4Linear(block_size, col_wise, scale_only, weights)
+    assert np.array_equal(to_np(layer.q_weights), oracle.native_from_canonical(kat["canon_w"]))
+    ps, pz = oracle.prepack_meta_sm80(block_size, col_wise, in_features, out_features, kat["scales"], kat["zps"])
+    assert np.array_equal(to_np(layer.q_scales).view(np.uint16), ps.view(np.uint16).reshape(-1))
+    assert np.array_equal(to_np(layer.q_zp), pz.reshape(-1))
+    # activations on the 0.25 grid in [-4, 4]: every product and partial sum is exact, any summation order agrees
+    g = torch.Generator(device="cpu").manual_seed(5)
+    x = (torch.randint(-16, 17, (9, in_features), generator=g).to(torch.float32) * 0.25).to(torch.float16)
+    y = layer(x.to(device))
+    ref = oracle.gemm(x.view(torch.int16).numpy().view(np.float16), kat["weights"])
+    assert np.array_equal(to_np(y).view(np.uint16), ref.view(np.uint16))
