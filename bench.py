@@ -46,6 +46,10 @@ CONFIGS = {
     "B16": (16, 8192, 28672, 64, True, "hbm"),
     "C4b": (2048, 4096, 4096, 64, True, "mfma"),
     "C2b": (1, 4096, 4096, 64, False, "hbm"),
+    "M256": (256, 4096, 4096, 64, True, "mfma"),
+    "M512": (512, 4096, 4096, 64, True, "mfma"),
+    "M768N11K": (768, 4096, 11008, 64, True, "mfma"),
+    "M256K11K": (256, 11008, 4096, 64, True, "mfma"),
 }
 BF16 = {"C4b", "C2b"}  # through blkq4_bf16_quant_sm80 / blkq4_bf16_gemm_sm80
 # every workload is replayed untimed for this long before the timed replays (a few milliseconds after an
@@ -67,6 +71,10 @@ DESCRIPTION = {
     "B16": "batch-16 decode on a wide layer M=16 K=8192 N=28672 bs64 asym (rows staged per slice)",
     "C4b": "C4 shape in bf16 (blkq4_bf16_gemm_sm80) M=2048 K=4096 N=4096 bs64 asym",
     "C2b": "C2 shape in bf16 (blkq4_bf16_gemm_sm80) M=1 K=4096 N=4096 bs64 sym",
+    "M256": "mid-size batch M=256 K=4096 N=4096 bs64 asym",
+    "M512": "mid-size batch M=512 K=4096 N=4096 bs64 asym",
+    "M768N11K": "ragged tile grid M=768 K=4096 N=11008 bs64 asym",
+    "M256K11K": "mid-size batch on a down projection M=256 K=11008 N=4096 bs64 asym (split tiles)",
 }
 
 
@@ -240,7 +248,7 @@ def check_and_baseline(name, a_dev, last_set, out_dev, w_host, with_cpu=True):
     if m <= 64:
         rows = np.arange(m)
     else:
-        want = 64 if m * n * k <= (1 << 36) else 12
+        want = m if m * n * k <= (1 << 35) else 64 if m * n * k <= (1 << 37) else 12
         rows = np.unique(np.concatenate([np.linspace(0, m - 1, want).astype(np.int64), [0, m - 1]]))
     a_rows = np.ascontiguousarray(a[rows])
     t0 = time.perf_counter()
@@ -300,6 +308,7 @@ def bench_gemm(torch, capi, name, device, steps, warmup, with_cpu=True):
     res = {
         "workload": DESCRIPTION[name], "value": round(value, 3), "unit": unit,
         "ms_per_step": round(per_call_wall * 1e3, 6), "kernel_us": round(per_call_evt * 1e6, 3),
+        "kernel": capi.gemm_plan(bs, col, m, n, k, has_offsets, name in BF16)[2],
         "timing": mode, "launches_per_region": n_launch, "weight_sets": copies,
         "weight_footprint_bytes": copies * per_set, "flops": flops, "bytes": nbytes,
         "tflops": round(flops / per_call_evt / 1e12, 3), "gbps": round(nbytes / per_call_evt / 1e9, 3),
@@ -450,7 +459,7 @@ def main(argv=None) -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r,C2r,M128,V128K,B16,C4b,C2b")
+    ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r,C2r,M128,M256,M512,M768N11K,M256K11K,V128K,B16,C4b,C2b")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-context", action="store_true", help="skip the floors and the library comparison")
     args = ap.parse_args(argv)

@@ -22,6 +22,7 @@ EXPORTED_SYMBOLS = (
     "blkq4_fp16_repack_sm80",
     "blkq4_bf16_quant_sm80",
     "blkq4_bf16_gemm_sm80",
+    "blkq4_gemm_plan_sm80",
     "blkq4_error_message_create",
     "blkq4_error_message_cstr",
     "blkq4_error_message_destroy",
@@ -65,6 +66,9 @@ def load() -> ctypes.CDLL:
     L.blkq4_bf16_quant_sm80.restype = i
     L.blkq4_bf16_gemm_sm80.argtypes = L.blkq4_fp16_gemm_bias_sm80.argtypes
     L.blkq4_bf16_gemm_sm80.restype = i
+    u64p = ctypes.POINTER(ctypes.c_uint64)
+    L.blkq4_gemm_plan_sm80.argtypes = [i, b, b, b, i, i, i, u64p, u64p, ctypes.c_char_p, sz, vp]
+    L.blkq4_gemm_plan_sm80.restype = i
     L.blkq4_error_message_create.restype = vp
     L.blkq4_error_message_cstr.argtypes = [vp]
     L.blkq4_error_message_cstr.restype = ctypes.c_char_p
@@ -179,3 +183,16 @@ def repack(to_sm80: bool, rows: int, columns: int, src, dst, stream=None):
     rc = L.blkq4_fp16_repack_sm80(int(to_sm80), rows, columns, _stream_ptr(stream), _ptr(src), _nbytes(src),
                                   _ptr(dst), _nbytes(dst), err.h)
     _check(rc, err)
+
+
+def gemm_plan(block_size: int, column_wise: bool, m: int, n: int, k: int, has_offsets: bool = True, bf16: bool = False):
+    """``blkq4_gemm_plan_sm80``: which kernel a GEMM of this shape runs, without running it (host-only).
+    -> (chosen_id, launched_id, description)."""
+    L = load()
+    err = _ErrMsg(L)
+    chosen, launched = ctypes.c_uint64(0), ctypes.c_uint64(0)
+    text = ctypes.create_string_buffer(256)
+    rc = L.blkq4_gemm_plan_sm80(block_size, column_wise, bf16, has_offsets, m, n, k, ctypes.byref(chosen),
+                                ctypes.byref(launched), text, len(text), err.h)
+    _check(rc, err)
+    return chosen.value, launched.value, text.value.decode()

@@ -9,6 +9,7 @@
 #include <cstdint>
 #include <string>
 
+#include "blkq4_choose.h"
 #include "blkq4_device.h"
 
 #define BLKQ4_EXPORT __attribute__((visibility("default")))
@@ -17,49 +18,6 @@ namespace {
 
 inline void set_error(std::string* err, std::string&& text) {
   if (err) *err = std::move(text);
-}
-
-// Which kernel multiplies m rows.  The reference switches at m > 16 (src/blkq4_f16_gemm_sm80.cu:343,
-// f16_gemm_sm80.h:63-72).  Here the weight-streaming kernel keeps going, in row groups of 32, for as long as
-// it is expected to be faster than the tile kernel, whose grid cannot fill the chip when m is small.
-// Both estimates are fits to measurements on MI355X: the streaming kernel's time grows with
-// row groups x n x k (2.8 us per row group at n = k = 4096) and, once it has more workgroups than compute
-// units, with whole rounds of them; the tile kernel runs its k / 64 steps once per round of 256 workgroups,
-// 0.64 us a step with 128 x 256 tiles, 0.42 us with the 128 x 128 tiles it uses when those cover the problem
-// in one round and 0.32 to 0.43 us (96 to 256 workgroups) with 64 x 128 tiles when even those do.
-inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k) {
-  if (m <= 16) return true;
-  if (m <= 32) {
-    // 17 to 32 rows: the streaming kernel wins unless it cannot keep the rows in LDS for all of K (it then
-    // fetches them again for every column group) and the problem is wide enough for the tile kernel's 32-row
-    // tiles to fill the chip: M = 32, K = 4096, N = 28672 takes 27.3 us streaming and 23.1 us in tiles, with
-    // N = 65536 53.7 and 39.5 us.
-    const bool rows_fit = 32L * k * 2 <= 160 * 1024;
-    return !column_wise || rows_fit || n / 128 < 224;
-  }
-  if (m > 1024) return false;
-  const long row_groups = (m + 31) / 32;
-  // blocks along N: the streaming kernel converts with 23 instead of 13 instructions per 8 weights
-  double streaming_us = (column_wise ? 2.8 : 5.6) * static_cast<double>(row_groups) * (static_cast<double>(n) / 4096.0) *
-                        (static_cast<double>(k) / 4096.0);
-  {
-    // its workgroups take 4, 2 or 1 column tiles of 16 (blocks along N: 1), as blkq4_skinny.hip chooses them
-    const long tiles = static_cast<long>(n / 16) * row_groups;
-    const long per_group = !column_wise ? 1 : tiles >= 640 ? 4 : tiles >= 320 ? 2 : 1;
-    const long streaming_groups = row_groups * ((n / 16 + per_group - 1) / per_group);
-    if (streaming_groups > 256) {
-      streaming_us *= static_cast<double>((streaming_groups + 255) / 256) / (static_cast<double>(streaming_groups) / 256.0);
-    }
-  }
-  const long smallest_tiles = static_cast<long>((m + 63) / 64) * ((n + 127) / 128);
-  const long small_tiles = static_cast<long>((m + 127) / 128) * ((n + 127) / 128);
-  const long workgroups = static_cast<long>((m + 127) / 128) * ((n + 255) / 256);
-  // (up to 64 rows the tile kernel has 64 x 256 tiles only: few workgroups, 0.55 us a step)
-  const double tile_us = (m <= 64) ? (k / 64) * 0.55
-                         : (smallest_tiles <= 256) ? (k / 64) * (0.25 + 0.0007 * static_cast<double>(smallest_tiles))
-                         : (small_tiles <= 256) ? (k / 64) * 0.42
-                                                : static_cast<double>((workgroups + 255) / 256) * (k / 64) * 0.64;
-  return streaming_us < tile_us;
 }
 
 inline bool supported_block_size(int bs) { return bs == 16 || bs == 32 || bs == 64; }
@@ -227,7 +185,8 @@ namespace {
 int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int n, int k, void* stream, void const* act_ptr,
                size_t a_size, void const* weights_ptr, size_t weights_size, void const* scales_ptr,
                size_t scales_size, void const* offsets_ptr, size_t offsets_size, void const* bias_ptr,
-               size_t bias_size, void* output_ptr, size_t output_size, void* err_msg_ptr) {
+               size_t bias_size, void* output_ptr, size_t output_size, void* err_msg_ptr,
+               blkq4::Choice* plan_out = nullptr) {
   auto* err = static_cast<std::string*>(err_msg_ptr);
   if (!supported_block_size(block_size)) {
     set_error(err, "Unsupported block size: " + std::to_string(block_size));
@@ -321,8 +280,28 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
   args.c = output_ptr;
   args.bias = has_bias ? bias_ptr : nullptr;
   args.stream = stream;
-  // The reference switches kernels at m > 16 (src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).
-  const bool streaming = streaming_kernel_takes(column_wise_blocking, m, n, k);
+  // Which kernel, in which shape (blkq4_choose.h; the reference switches at m > 16,
+  // src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).  A split tile kernel needs a workspace: the
+  // library's own for this stream; when there is none to be had (out of memory, too many streams), the plan is
+  // made again without one.
+  blkq4::Choice choice = blkq4::choose(column_wise_blocking, m, n, k, blkq4_dev_workspace_capacity());
+  if (plan_out != nullptr) {
+    *plan_out = choice;
+    return 0;
+  }
+  if (choice.family == blkq4::kFamilyTile && choice.t.split_k > 1) {
+    void* workspace = nullptr;
+    if (int code = blkq4_dev_workspace(stream, &workspace)) return device_failure(code, err);
+    if (workspace == nullptr) {
+      choice = blkq4::choose(column_wise_blocking, m, n, k, 0);
+    } else {
+      args.workspace = workspace;
+      args.workspace_bytes = blkq4_dev_workspace_capacity();
+    }
+  }
+  args.streaming = choice.s;
+  args.tile = choice.t;
+  const bool streaming = choice.family == blkq4::kFamilyStreaming;
   const int code = bf16 ? (streaming ? blkq4_dev_skinny_bf16(&args) : blkq4_dev_gemm_bf16(&args))
                         : (streaming ? blkq4_dev_skinny(&args) : blkq4_dev_gemm(&args));
   if (code) return device_failure(code, err);
@@ -370,6 +349,75 @@ extern "C" BLKQ4_EXPORT int blkq4_bf16_gemm_sm80(int block_size, bool column_wis
   return gemm_entry(true, block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr,
                     weights_size, scales_ptr, scales_size, offsets_ptr, offsets_size, bias_ptr, bias_size,
                     output_ptr, output_size, err_msg_ptr);
+}
+
+// Which kernel a GEMM of this shape runs, without running it: the identity of the kernel blkq4::choose() picks
+// and the identity of the instantiation the launcher maps that choice to (they must agree), plus a description.
+extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wise_blocking, bool bf16,
+                                                 bool has_offsets, int m, int n, int k, uint64_t* chosen_id,
+                                                 uint64_t* launched_id, char* description,
+                                                 size_t description_size, void* err_msg_ptr) {
+  auto* err = static_cast<std::string*>(err_msg_ptr);
+  if (!supported_block_size(block_size)) {
+    set_error(err, "Unsupported block size: " + std::to_string(block_size));
+    return -1;
+  }
+  const int krow = column_wise_blocking ? block_size : 1;
+  const int kcol = column_wise_blocking ? 1 : block_size;
+  if (m <= 0 || n <= 0 || k <= 0) {
+    set_error(err, "Empty problem size: " + std::to_string(m) + "x" + std::to_string(n) + "x" + std::to_string(k));
+    return -1;
+  }
+  if ((k % 64) != 0 || (k % krow) != 0 || (n % kcol) != 0 || (n % 32) != 0) {
+    set_error(err, "Kernel execution failed: Error Invalid Problem");
+    return -1;
+  }
+  const blkq4::Choice choice = blkq4::choose(column_wise_blocking, m, n, k, blkq4_dev_workspace_capacity());
+  blkq4_gemm_args args{};
+  args.block_size = block_size;
+  args.column_wise = column_wise_blocking ? 1 : 0;
+  args.m = m;
+  args.n = n;
+  args.k = k;
+  // addresses that are never used: the launchers only look at their alignment
+  void* const dummy = reinterpret_cast<void*>(uintptr_t{1} << 20);
+  args.a = args.packed_w = args.scales = dummy;
+  args.zero_points = has_offsets ? dummy : nullptr;
+  args.c = dummy;
+  args.streaming = choice.s;
+  args.tile = choice.t;
+  args.dry_run = 1;
+  uint64_t launched = 0;
+  args.launched_id = &launched;
+  const bool streaming = choice.family == blkq4::kFamilyStreaming;
+  const int code = bf16 ? (streaming ? blkq4_dev_skinny_bf16(&args) : blkq4_dev_gemm_bf16(&args))
+                        : (streaming ? blkq4_dev_skinny(&args) : blkq4_dev_gemm(&args));
+  if (code) return device_failure(code, err);
+  if (chosen_id != nullptr) *chosen_id = blkq4::choice_id(choice);
+  if (launched_id != nullptr) *launched_id = launched;
+  if (description != nullptr && description_size > 0) {
+    std::string text;
+    if (streaming) {
+      const auto& p = choice.s;
+      text = "streaming: " + std::to_string(p.waves) + " waves" + (p.split == 1 ? " with column tiles of their own" : " splitting K") +
+             ", " + std::to_string(p.nt) + " column tile(s) x " + std::to_string(16 * p.mt) + " rows, " +
+             std::to_string(p.depth) + " slices in flight, rows " +
+             (p.am == blkq4::kRowsWholeInLds ? "whole in LDS" : "staged per slice") + ", " + std::to_string(p.row_groups) +
+             " row group(s), " + std::to_string(p.grid) + " workgroups" + (p.refill ? " (walking)" : "");
+    } else {
+      const auto& t = choice.t;
+      text = "tile: " + std::to_string(32 * t.rt * t.wm) + " x " + std::to_string(32 * t.nt * t.wn) + ", " +
+             std::to_string(t.wm * t.wn) + " + " + std::to_string(t.pw) + " waves, " + std::to_string(t.tiles) + " tiles";
+      if (t.split_k > 1) {
+        text += ", the last " + std::to_string(t.split_tiles) + " in " + std::to_string(t.split_k) + " parts (workspace " +
+                std::to_string(t.workspace_bytes) + " bytes)";
+      }
+    }
+    const size_t len = text.size() < description_size - 1 ? text.size() : description_size - 1;
+    text.copy(description, len);
+    description[len] = '\0';
+  }
+  return 0;
 }
 
 extern "C" BLKQ4_EXPORT int blkq4_fp16_repack_sm80(int to_sm80, int rows, int columns, void* stream,

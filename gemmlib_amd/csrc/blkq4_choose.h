@@ -1,0 +1,384 @@
+// Which kernel multiplies a given problem, and in which shape: the ONE place where the thresholds live.
+// Host-only, plain C++ (no HIP headers): blkq4_api.cpp asks blkq4::choose(), hands the answer to the launchers
+// inside blkq4_gemm_args, and the launchers (blkq4_gemm.hip, blkq4_skinny.hip) map it to a kernel instantiation
+// without any threshold of their own.
+//
+// The reference switches kernels at m > 16 and knows two tile shapes (src/blkq4_f16_gemm_sm80.cu:343,
+// src/mickey/blk_q4/f16_gemm_sm80.h:63-72); everything below is this library's own cost model, fitted to
+// measurements on MI355X.
+
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "blkq4_device.h"
+
+namespace blkq4 {
+
+constexpr int kComputeUnits = 256;
+constexpr size_t kMaxLdsBytes = 160 * 1024;
+constexpr int kStreamingMaxRows = 1024;
+
+// Where the streaming kernel's waves find their activation fragments.
+constexpr int kRowsWholeInLds = 1;    // all rows, all of K, staged once per workgroup
+constexpr int kRowsPerSlotInLds = 2;  // 16 * MT rows x 128 k staged per slot, private to the wave
+
+constexpr int kFamilyStreaming = 0;  // weight-streaming kernel (blkq4_skinny.hip)
+constexpr int kFamilyTile = 1;       // MFMA tile kernel (blkq4_gemm.hip)
+
+using StreamingShape = blkq4_streaming_plan;  // see blkq4_device.h
+using TileShape = blkq4_tile_plan;
+
+struct Choice {
+  int family;
+  StreamingShape s;
+  TileShape t;
+};
+
+// A kernel's identity as one number: what choose() picked and what a launcher started can be compared.
+inline uint64_t streaming_id(int depth, int nt, int mt, int waves, int am, int split, bool refill) {
+  return 1ull << 60 | static_cast<uint64_t>(depth) << 40 | static_cast<uint64_t>(nt) << 32 |
+         static_cast<uint64_t>(mt) << 24 | static_cast<uint64_t>(waves) << 16 | static_cast<uint64_t>(am) << 12 |
+         static_cast<uint64_t>(split) << 4 | (refill ? 1u : 0u);
+}
+inline uint64_t tile_id(int rt, int nt, int wm, int wn, int pw, bool split) {
+  return 2ull << 60 | static_cast<uint64_t>(rt) << 40 | static_cast<uint64_t>(nt) << 32 |
+         static_cast<uint64_t>(wm) << 24 | static_cast<uint64_t>(wn) << 16 | static_cast<uint64_t>(pw) << 8 |
+         (split ? 1u : 0u);
+}
+inline uint64_t choice_id(const Choice& c) {
+  return c.family == kFamilyStreaming
+             ? streaming_id(c.s.depth, c.s.nt, c.s.mt, c.s.waves, c.s.am, c.s.split, c.s.refill != 0)
+             : tile_id(c.t.rt, c.t.nt, c.t.wm, c.t.wn, c.t.pw, c.t.split_k > 1);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Streaming kernel
+// ---------------------------------------------------------------------------------------------------------
+
+// Slices that `waves` waves with rings of `depth` slices request for one column group: every wave asks for
+// whole rings, also when it has fewer slices left.
+inline int requested_slices(int k, int waves, int depth) {
+  const int slices = (k / 32 + 3) / 4;
+  int total = 0;
+  for (int w = 0; w < waves; ++w) {
+    const int mine = (slices - w + waves - 1) / waves;
+    total += (mine + depth - 1) / depth * depth;
+  }
+  return total;
+}
+
+// The kernel is bound by instruction issue as much as by the weight stream, so what matters is how
+// evenly the workgroups fill the 256 compute units: with T column tiles per workgroup the busiest
+// unit works through ceil(workgroups / 256) * T tiles.  Wider workgroups also re-read the activation
+// rows less often, which weighs more the more rows there are.
+inline void streaming_tiles_per_workgroup(int m, int n, int k, int* nt, int* depth) {
+  const int tiles = n / 16;
+  // cost of fetching the activation rows relative to one tile's work: small while they are staged once per
+  // workgroup; when K is too long for that they are fetched again for every column group, 16 rows x 2 bytes
+  // against a tile's 16 columns x 1/2 byte per k
+  int rows = 1;
+  while (rows < m) rows *= 2;
+  const bool rows_fit = static_cast<size_t>(rows) * static_cast<size_t>(k) * 2 <= kMaxLdsBytes;
+  const float a_weight = !rows_fit ? static_cast<float>(rows) / 4.0f : (m > 4) ? 0.2f : 0.05f;
+  float best = 0.f;
+  *nt = 1;
+  for (int t = 1; t <= 3; ++t) {
+    const int wgs = (tiles + t - 1) / t;
+    const int rounds = (wgs + kComputeUnits - 1) / kComputeUnits;
+    const float cost = static_cast<float>(rounds) * (static_cast<float>(t) + a_weight);
+    if (t == 1 || cost < best) {
+      best = cost;
+      *nt = t;
+    }
+  }
+  // one tile per workgroup: 8 slices in flight while at most two workgroups share a unit, else 4
+  // (the deeper ring needs too many registers for more resident waves)
+  *depth = (*nt == 1 && tiles <= 2 * kComputeUnits) ? 8 : 4;
+}
+
+// Launch geometry of one instantiation.  Many more workgroups than the chip holds at once: a workgroup then
+// walks over several column groups (cg, cg + cg_stride, ...) and requests the first slices of the next one
+// while it finishes the current one, so only the first column group of a workgroup waits for its weights with
+// nothing else to do.  The partial tiles then get LDS of their own: the rows stay where they are for the next
+// column group.  (not the sixteen-wave kernel for blocks along N: its walking variant does not fit in 128
+// registers)
+inline void streaming_geometry(StreamingShape* s, bool row, int n, int k) {
+  constexpr int kPersistentFactor = 2;  // column groups per workgroup from which on workgroups walk
+  const size_t red_bytes = (s->split == 1) ? 0 : static_cast<size_t>(s->waves) * s->nt * s->mt * 64 * 4 * 4;
+  const size_t per_slot_bytes = static_cast<size_t>(s->waves) * s->depth * 16 * s->mt * 256;
+  // the rows are copied 1 KiB at a time; the partial tiles of the reduction reuse their space
+  const size_t a_bytes = s->am == kRowsWholeInLds
+                             ? ((((static_cast<size_t>(k) * 2) << s->rows_log2) + 1023) & ~size_t{1023})
+                             : per_slot_bytes;
+  const int group_tiles = s->nt * (s->waves / s->split);
+  const int col_groups = (n / 16 + group_tiles - 1) / group_tiles;
+  int cg_stride = (col_groups + 31) / 32 * 32;  // one column group per workgroup
+  size_t lds_bytes = a_bytes > red_bytes ? a_bytes : red_bytes;
+  size_t red_offset = 0;
+  const bool may_walk = !(row && s->waves == 16);
+  if (may_walk && a_bytes + red_bytes <= kMaxLdsBytes) {
+    const int by_lds = static_cast<int>(kMaxLdsBytes / (a_bytes + red_bytes));
+    const int by_waves = 32 / s->waves;
+    const int resident = kComputeUnits * (by_lds < by_waves ? by_lds : by_waves);
+    int stride = (resident / s->row_groups) / 32 * 32;
+    if (stride < 32) stride = 32;
+    if (cg_stride >= kPersistentFactor * stride) {
+      cg_stride = stride;
+      lds_bytes = a_bytes + red_bytes;
+      red_offset = a_bytes;
+    }
+  }
+  s->cg_stride = cg_stride;
+  s->grid = static_cast<uint32_t>(cg_stride) * static_cast<uint32_t>(s->row_groups);
+  s->lds_bytes = static_cast<uint32_t>(lds_bytes);
+  s->red_offset = static_cast<uint32_t>(red_offset);
+  // workgroups walk over several column groups, or waves stream all of K by themselves
+  s->refill = (cg_stride < col_groups || s->split == 1) ? 1 : 0;
+}
+
+inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
+  StreamingShape s{};
+  auto set = [&](int depth, int nt, int mt, int waves, int am, int split) {
+    s.depth = depth; s.nt = nt; s.mt = mt; s.waves = waves; s.am = am; s.split = split;
+  };
+  s.row_groups = 1;
+  if (m > 16) {
+    // Row groups of 32 rows (two row tiles share one conversion of the weights), eight waves.  Every workgroup
+    // fetches the 32 rows of its group for all of K, so wide workgroups (more column tiles) mean less
+    // activation traffic; but there should be a workgroup for most compute units (measured: four tiles per
+    // workgroup from 160 workgroups of four on, two from 160 of two on).  Blocks along N: 28 registers of
+    // packed weights, scales and zero-points per slot and tile, so one tile.
+    s.row_groups = (m + 31) / 32;
+    s.rows_log2 = 5;
+    const long tiles = static_cast<long>(n / 16) * s.row_groups;
+    const int nt = row ? 1 : tiles >= 640 ? 4 : tiles >= 320 ? 2 : 1;
+    const bool rows_fit = static_cast<size_t>(k) * 2 * 32 <= kMaxLdsBytes;
+    set(2, nt, 2, 8, rows_fit ? kRowsWholeInLds : kRowsPerSlotInLds, 8);
+    streaming_geometry(&s, row, n, k);
+    return s;
+  }
+  while ((1 << s.rows_log2) < m) ++s.rows_log2;
+  const size_t a_bytes = (((static_cast<size_t>(k) * 2) << s.rows_log2) + 1023) & ~size_t{1023};
+  const bool rows_fit = a_bytes <= kMaxLdsBytes;
+  const int tiles = n / 16;
+  const int slices = (k / 32 + 3) / 4;
+  auto done = [&]() {
+    streaming_geometry(&s, row, n, k);
+    return s;
+  };
+  {
+    // Enough column tiles to give every wave the chip can hold one of its own, and rows small enough for
+    // several workgroups per compute unit: the waves do not split K, each streams all of K for its own tile:
+    // no sums across waves, no barriers, and a ring that stays full from the first slice to the last.
+    // Break-even measured against workgroups that split K and walk (blocks along N gain more: their
+    // sixteen-wave kernel has no walking variant); from 832 tiles on when K is no multiple of what the
+    // splitting waves' rings hold, which then ask for a fifth more slices than there are (K = 5120,
+    // N = 13824: 14.5 -> 12.7 us).  Four slices in flight per wave: with eight the kernel needs 90 registers
+    // and a SIMD holds five waves instead of seven (52 against 55 us at N = 128256).
+    const size_t max_row_bytes = (row ? 32 : 16) * 1024;
+    const bool rings_fit_k =
+        5 * requested_slices(k, 16, 2) < 6 * slices || 5 * requested_slices(k, 8, 4) < 6 * slices;
+    const int min_tiles = row ? 896 : rings_fit_k ? 2000 : 832;
+    if (tiles >= min_tiles && a_bytes <= max_row_bytes) {
+      set(4, 1, 1, 4, kRowsWholeInLds, 1);
+      return done();
+    }
+  }
+  if (!row && (!rows_fit || m > 4) && k >= 1024) {
+    // Wide N and more than four rows, or K too long for the rows to stay in LDS: the rows are staged per
+    // slice, a workgroup takes four column tiles (the rows are fetched again for every column group) and a
+    // wave keeps two slices in flight, so that the slots are small enough for several workgroups per compute
+    // unit: eight waves from 832 column tiles on, four from 1536 on.  Measured against every other shape of
+    // workgroup: M = 16, K = 8192: N = 14336 24.3 -> 17.6 us, N = 28672 43.1 -> 34.1 us; rows that would fit
+    // (M = 16, K = 4096, N = 14336: 13.2 -> 11.1 us) gain less or nothing, never lose more than 3 %.
+    if (tiles >= 1536) {
+      set(2, 4, 1, 4, kRowsPerSlotInLds, 4);
+      return done();
+    }
+    if (tiles >= 832) {
+      set(2, 4, 1, 8, kRowsPerSlotInLds, 8);
+      return done();
+    }
+  }
+  int nt, depth;
+  streaming_tiles_per_workgroup(m, n, k, &nt, &depth);
+  if (row) nt = 1;
+  if (nt > 1) depth = 4;
+  if (k >= 4096 && rows_fit) {
+    // sixteen waves when there is enough K: each wave has less to convert after its last load has arrived,
+    // and more of that work overlaps the loads of the other waves.  With more workgroups than compute units,
+    // eight waves: smaller workgroups fill the units more evenly (M = 1, K = 4096, N = 14336: 11.4 -> 9.5 us),
+    // unless their rings would ask for many more slices than K has.
+    const int d8 = depth > 4 ? 4 : depth;
+    const int col_groups = (tiles + nt - 1) / nt;
+    if (!row && col_groups > kComputeUnits && 20 * requested_slices(k, 8, d8) <= 21 * requested_slices(k, 16, 2)) {
+      set(d8, nt, 1, 8, kRowsWholeInLds, 8);
+    } else {
+      set(2, nt, 1, 16, kRowsWholeInLds, 16);
+    }
+    return done();
+  }
+  if (k >= 1024) {
+    set(depth > 4 ? 4 : depth, nt, 1, 8, rows_fit ? kRowsWholeInLds : kRowsPerSlotInLds, 8);  // 8 * 4 * 4 KiB of rows
+    return done();
+  }
+  set(depth, nt, 1, 4, kRowsWholeInLds, 4);  // K < 1024: at most 32 KiB of rows
+  return done();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Tile kernel
+// ---------------------------------------------------------------------------------------------------------
+
+inline long ceil_div(long a, long b) { return (a + b - 1) / b; }
+
+// The tile shapes, (rt, nt, wm, wn, pw): 64 x 128, 128 x 128 and 128 x 256 tiles of four computing waves
+// (64 x 32, 128 x 32, 128 x 64 each) plus four producer waves that only issue copies, and 256 x 256 tiles of
+// four waves of 256 x 64 (every register of a SIMD belongs to the one wave, which leaves no room for producer
+// waves).  Larger tiles convert fewer weights per MFMA; smaller ones fill the chip with smaller problems.
+constexpr int kTileShapes[4][5] = {{2, 1, 1, 4, 4}, {4, 1, 1, 4, 4}, {4, 2, 1, 4, 4}, {8, 2, 1, 4, 0}};
+
+// Arrival counters first (one per split tile), then the fp32 partial tiles of the split tiles.
+constexpr size_t kCounterBytes = 16 * 1024;  // room for 4096 split tiles
+constexpr int kMinKTilesPerPart = 4;         // a part of a split tile is at least this many 64-deep k tiles
+constexpr int kMaxSplit = 4;                 // the workgroup that arrives last reads all the parts by itself
+
+inline size_t tile_workspace_bytes(const TileShape& t) {
+  if (t.split_k <= 1) return 0;
+  const size_t tile_elems = static_cast<size_t>(32 * t.rt * t.wm) * (32 * t.nt * t.wn);
+  return kCounterBytes + static_cast<size_t>(t.split_tiles) * t.split_k * tile_elems * 4;
+}
+
+// Measured microseconds per 64-deep k tile of one workgroup when `busy` workgroups share the chip (fp16, blocks
+// of 64 along K, K = N = 4096 ... 11008): flat while half the compute units idle, then rising with the load
+// on the memory system and the clock the chip holds -- 64 x 128: 0.29 (<= 192 workgroups) to 0.36 (256),
+// 128 x 128: 0.37 (<= 128) to 0.575, 128 x 256: 0.65 (<= 128) to 0.945, 256 x 256: 1.2 (<= 128) to 1.72 --
+// and what a workgroup spends outside its main loop.
+struct TileCost {
+  double step_idle, step_slope, fixed;
+  int flat_until;
+};
+inline TileCost tile_cost(const TileShape& t) {
+  if (t.rt == 8) return {1.20, 0.0041, 3.0, 128};
+  if (t.rt == 4 && t.nt == 2) return {0.65, 0.0023, 2.0, 128};
+  if (t.rt == 4) return {0.37, 0.0016, 1.5, 128};
+  if (t.rt == 2 && t.wn == 4) return {0.29, 0.0011, 1.0, 192};
+  return {0.55, 0.0, 0.0, 256};  // tiles of one row tile (up to 64 rows)
+}
+inline double tile_round_us(const TileShape& t, int k_tiles, long busy) {
+  const TileCost c = tile_cost(t);
+  const long b = busy < kComputeUnits ? busy : kComputeUnits;
+  return c.fixed + k_tiles * (c.step_idle + (b > c.flat_until ? (b - c.flat_until) * c.step_slope : 0.0));
+}
+
+// Estimated time of the tile kernel with shape t (split or not) on k: whole rounds of unsplit tiles, a last
+// round of what is left of them, then one round of parts: their share of the k tiles, the partial tile
+// written once and all parts read by the workgroup that arrives last (about 100 GB/s) plus 4 us for the cache
+// write-back and invalidate and the two extra barriers (measured: 64 x 128 in 2 parts 17.7 - 19.1 us against
+// 18.7 unsplit at M = 256, K = N = 4096; 128 x 128 in 3 parts 32.7 against 44.6 us at K = 11008).
+inline double tile_estimate_us(const TileShape& t, int k) {
+  const int kt = k / 64;
+  const long whole = t.tiles - (t.split_k > 1 ? t.split_tiles : 0);
+  double us = static_cast<double>(whole / kComputeUnits) * tile_round_us(t, kt, kComputeUnits);
+  if (whole % kComputeUnits) us += tile_round_us(t, kt, whole % kComputeUnits);
+  if (t.split_k > 1) {
+    const long units = static_cast<long>(t.split_tiles) * t.split_k;
+    const double tile_bytes = 4.0 * (32 * t.rt * t.wm) * (32 * t.nt * t.wn);
+    us += static_cast<double>(ceil_div(units, kComputeUnits)) *
+          (tile_round_us(t, static_cast<int>(ceil_div(kt, t.split_k)), units) + 4.0 + (1 + t.split_k) * tile_bytes / 100e3);
+  }
+  return us;
+}
+
+// The tile kernel's plan: the shape with the smallest estimate; when its last round of tiles would leave most
+// of the chip idle and the estimate says it pays, those last `split_tiles` tiles are each shared out over
+// split_k workgroups.  Up to 64 rows with blocks along K: tiles of one row tile, which fetch every packed
+// weight once (128 columns with four waves and four producer waves when such tiles fill the chip in one
+// round, else 256 columns with eight waves; M = 64, K = 4096, N = 28672: 34.7 against 26.3 us).
+inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspace_capacity) {
+  TileShape best{};
+  auto shape = [&](int rt, int nt, int wm, int wn, int pw) {
+    TileShape t{};
+    t.rt = rt; t.nt = nt; t.wm = wm; t.wn = wn; t.pw = pw;
+    t.split_k = 1;
+    t.tiles = static_cast<int>(ceil_div(m, 32 * rt * wm) * ceil_div(n, 32 * nt * wn));
+    return t;
+  };
+  if (column_wise && m <= 64) {
+    const bool one_round_of_128 = n / 128 >= 224 && n / 128 <= kComputeUnits;
+    const int rt = m <= 32 ? 1 : 2;
+    return one_round_of_128 ? shape(rt, 1, 1, 4, 4) : shape(rt, 1, 1, 8, 0);
+  }
+  const int kt = k / 64;
+  double best_us = 0.0, best_unsplit_us = 0.0;
+  for (const auto& sh : kTileShapes) {
+    const TileShape t = shape(sh[0], sh[1], sh[2], sh[3], sh[4]);
+    const double us = tile_estimate_us(t, k);
+    if (best.rt == 0 || us < best_us) {
+      best = t;
+      best_us = us;
+    }
+  }
+  best_unsplit_us = best_us;
+  for (const auto& sh : kTileShapes) {
+    TileShape t = shape(sh[0], sh[1], sh[2], sh[3], sh[4]);
+    const int rem = t.tiles % kComputeUnits;
+    if (rem == 0) continue;
+    for (int split = 2; split <= kMaxSplit; ++split) {
+      if (rem * split > kComputeUnits || kt / split < kMinKTilesPerPart) break;
+      t.split_k = split;
+      t.split_tiles = rem;
+      t.workspace_bytes = tile_workspace_bytes(t);
+      if (t.workspace_bytes > workspace_capacity || static_cast<size_t>(rem) * sizeof(int) > kCounterBytes) continue;
+      const double us = tile_estimate_us(t, k);
+      // a split has to promise a tenth less than the best unsplit shape: its estimate is the less certain one
+      if (us < 0.9 * best_unsplit_us && us < best_us) {
+        best = t;
+        best_us = us;
+      }
+    }
+  }
+  return best;
+}
+
+// Which kernel multiplies m rows.  The reference switches at m > 16 (src/blkq4_f16_gemm_sm80.cu:343,
+// f16_gemm_sm80.h:63-72).  Here the weight-streaming kernel keeps going, in row groups of 32, for as long as
+// it is expected to be faster than the tile kernel, whose grid cannot fill the chip when m is small.
+// The streaming kernel's time grows with row groups x n x k (2.8 us per row group at n = k = 4096) and, once
+// it has more workgroups than compute units, with whole rounds of them.
+inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const StreamingShape& s, double tile_us) {
+  if (m <= 16) return true;
+  if (m <= 32) {
+    // 17 to 32 rows: the streaming kernel wins unless it cannot keep the rows in LDS for all of K (it then
+    // fetches them again for every column group) and the problem is wide enough for the tile kernel's 32-row
+    // tiles to fill the chip: M = 32, K = 4096, N = 28672 takes 27.3 us streaming and 23.1 us in tiles, with
+    // N = 65536 53.7 and 39.5 us.
+    const bool rows_fit = 32L * k * 2 <= static_cast<long>(kMaxLdsBytes);
+    return !column_wise || rows_fit || n / 128 < 224;
+  }
+  if (m > kStreamingMaxRows) return false;
+  const long row_groups = s.row_groups;
+  // blocks along N: the streaming kernel converts with 23 instead of 13 instructions per 8 weights
+  double streaming_us = (column_wise ? 2.8 : 5.6) * static_cast<double>(row_groups) * (static_cast<double>(n) / 4096.0) *
+                        (static_cast<double>(k) / 4096.0);
+  const long streaming_groups = row_groups * ceil_div(n / 16, s.nt);
+  if (streaming_groups > kComputeUnits) {
+    streaming_us *= static_cast<double>(ceil_div(streaming_groups, kComputeUnits)) /
+                    (static_cast<double>(streaming_groups) / kComputeUnits);
+  }
+  return streaming_us < tile_us;
+}
+
+// The whole decision.  workspace_capacity: bytes of workspace the caller could hand to a split tile kernel
+// (0: none, no split).
+inline Choice choose(bool column_wise, int m, int n, int k, size_t workspace_capacity) {
+  Choice c{};
+  if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k);
+  c.t = tile_plan(column_wise, m, n, k, workspace_capacity);
+  c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_estimate_us(c.t, k)) ? kFamilyStreaming : kFamilyTile;
+  return c;
+}
+
+}  // namespace blkq4

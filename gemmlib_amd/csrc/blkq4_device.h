@@ -47,6 +47,29 @@ typedef struct {
   int bf16;            /* 1: src and scales are bf16; 0: fp16 */
 } blkq4_prepack_args;
 
+/* Which streaming kernel runs and how it is launched: the template parameters of skinny_mfma_kernel
+ * (blkq4_skinny.hip) and the launch geometry derived from them.  Filled in by blkq4::choose() (blkq4_choose.h). */
+typedef struct {
+  int depth, nt, mt, waves, am, split; /* split = waves (the waves split K) or 1 (they do not) */
+  int rows_log2, row_groups;
+  int refill;          /* workgroups walk over several column groups / waves stream all of K by themselves */
+  int cg_stride;       /* column groups a workgroup steps over */
+  uint32_t grid;       /* workgroups */
+  uint32_t lds_bytes;  /* dynamic LDS */
+  uint32_t red_offset; /* where the partial tiles of the sum across waves lie in it */
+} blkq4_streaming_plan;
+
+/* Which tile kernel runs: wm x wn computing waves of (32 rt) x (32 nt) outputs, pw producer waves.
+ * split_k > 1: the last split_tiles tiles of the tile order are computed by split_k workgroups each, which
+ * leave fp32 partial tiles in the workspace; the last of them to finish sums them in a fixed order. */
+typedef struct {
+  int rt, nt, wm, wn, pw;
+  int split_k;            /* 1: no workspace needed */
+  int split_tiles;        /* 0 without a split */
+  int tiles;              /* all tiles of the problem */
+  size_t workspace_bytes; /* arrival counters + partial tiles, 0 without a split */
+} blkq4_tile_plan;
+
 typedef struct {
   int block_size;
   int column_wise;          /* as in blkq4_prepack_args */
@@ -58,6 +81,12 @@ typedef struct {
   void* c;                  /* fp16 [m][n] */
   const void* bias;         /* fp16 [n] added to every row of c after its rounding to fp16, or NULL */
   void* stream;
+  blkq4_streaming_plan streaming; /* read by blkq4_dev_skinny* */
+  blkq4_tile_plan tile;           /* read by blkq4_dev_gemm* */
+  void* workspace;                /* tile.split_k > 1: device memory of workspace_bytes, 256-byte aligned, whose */
+  size_t workspace_bytes;         /* first 16 KiB (the arrival counters) are zero between launches */
+  int dry_run;                    /* 1: launch nothing, only report the kernel */
+  uint64_t* launched_id;          /* if not NULL: receives the identity of the kernel instantiation (blkq4_choose.h) */
 } blkq4_gemm_args;
 
 typedef struct {
@@ -75,6 +104,12 @@ int blkq4_dev_gemm_bf16(const blkq4_gemm_args* args);   /* the tile kernel with 
 int blkq4_dev_skinny_bf16(const blkq4_gemm_args* args); /* the same with bf16 a, scales, c and bias */
 int blkq4_dev_repack(const blkq4_repack_args* args);
 const char* blkq4_dev_error_string(int code);
+
+/* Workspace of the split tile kernels: the library-owned buffer of (current device, stream), allocated on first
+ * use with a fixed size and its counters zeroed; *ptr = NULL (and 0 returned) when there is none and none can be
+ * made (out of memory, or too many streams have one). */
+size_t blkq4_dev_workspace_capacity(void);
+int blkq4_dev_workspace(void* stream, void** ptr);
 
 #ifdef __cplusplus
 }

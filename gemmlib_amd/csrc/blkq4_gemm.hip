@@ -2,7 +2,7 @@
 // counts the weight-streaming kernel does not take.
 //
 // A workgroup is WM x WN computing waves, each owning (32*RT) x (32*NT) outputs, plus PW producer waves
-// that only issue copies (see launch_rt for the shapes in use: 256 x 256, 128 x 256, 128 x 128 and 64 x 128 tiles).
+// that only issue copies (see blkq4_choose.h for the shapes in use: 256 x 256, 128 x 256, 128 x 128 and 64 x 128 tiles).
 // A wave converts each of its NT 32-column weight fragments to fp16 once per 16-deep k step and feeds it
 // to RT MFMAs; a wave can issue about five VALU instructions in the shadow of one 32x32x16 MFMA, and the
 // conversion takes 13 per fragment and step.
@@ -46,6 +46,7 @@
 
 #include <stdint.h>
 
+#include "blkq4_choose.h"
 #include "blkq4_dequant.h"
 #include "blkq4_device.h"
 #include "blkq4_launch.h"
@@ -111,18 +112,27 @@ struct Stage {
   static constexpr int kMTotal = ROW ? kRowScaleOps + kRowZpOps : WN * kBlocks;
   static constexpr int kMOps = (kMTotal + kCopiers - 1) / kCopiers;
   static constexpr int kOps = kAOps + kBOps + kMOps;
-  // ring of k tiles in LDS, requested kDistance tiles ahead of the one being consumed
+  // ring of k tiles in LDS, requested kDistance tiles ahead of the one being consumed (deeper rings were
+  // measured and lose: up to eight slots, M = 256, K = N = 4096: 64 x 128 tiles 18.7 -> 20.4 us, 128 x 128 tiles
+  // 24.3 -> 28.3 us; C4 unchanged)
   static constexpr int kStages = (4 * kBytes <= 160 * 1024) ? 4 : 3;
   static constexpr int kDistance = kStages - 1;  // the slot being refilled is the one nobody reads
+  static_assert((kDistance - 1) * kOps <= 63, "more copies in flight than the counter holds");
 };
 
 // (BF repeats kBF so that the two compilations' kernels carry different names in a trace)
-template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW, bool BF = kBF>
+// SK: the last `split_tiles` tiles of the tile order are computed by `split_k` workgroups each (workgroup
+// whole_tiles + u: tile whole_tiles + u % split_tiles, part u / split_tiles of its k tiles).  Such a workgroup
+// leaves its fp32 partial tile in `partials` and counts itself in the tile's arrival counter; the one that
+// arrives last adds the parts up in the order 0, 1, ..., split_k - 1 (so the result does not depend on who
+// that is), clears the counter for the next launch and runs the epilogue.  Nobody waits for anybody.
+template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW, bool SK, bool BF = kBF>
 __global__ __launch_bounds__(64 * (WM * WN + PW))
     __attribute__((amdgpu_waves_per_eu((WM * WN + PW) / 4, (WM * WN + PW) / 4))) void gemm_mfma_kernel(
         const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ S,
         const uint8_t* __restrict__ Z, uint16_t* __restrict__ C, const uint16_t* __restrict__ bias, int M, int N,
-        int K, int m_tiles) {
+        int K, int m_tiles, int whole_tiles, int split_tiles, int split_k, float* __restrict__ partials,
+        int* __restrict__ counters) {
   using St = Stage<BS, RT, NT, WM, WN, PW, ROW>;
   constexpr int kComputeWaves = WM * WN;
   static_assert(!ROW || St::kGroups % 2 == 0, "scale copies take two column groups at a time");
@@ -152,15 +162,30 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   const int i = lane & 31;  // row of an activation fragment / column of a weight fragment
   const int h = lane >> 5;  // which 32-deep half of the 64-deep k tile this lane covers
 
-  const int bm = blockIdx.x % m_tiles;
-  const int bn = blockIdx.x / m_tiles;
+  int tile = blockIdx.x;
+  int part = 0;      // which share of the k tiles, of `parts`
+  int parts = 1;
+  if (SK && tile >= whole_tiles) {
+    const int u = tile - whole_tiles;
+    tile = whole_tiles + u % split_tiles;
+    part = u / split_tiles;
+    parts = split_k;
+  }
+  const int bm = tile % m_tiles;
+  const int bn = tile / m_tiles;
   const int m0 = bm * kBM;
   const int nw0 = bn * kBN + wn * (32 * NT);
   // N is a multiple of 32, so 32-column fragments are whole; a fragment past the end re-reads the last one
   int nbase[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) nbase[t] = min(nw0 + 32 * t, N - 32);
-  const int KT = K / kBK;
+  // this workgroup's k tiles: [kt_first, kt_first + KT)
+  const int kt_first = SK ? static_cast<int>(static_cast<long>(K / kBK) * part / parts) : 0;
+  const int KT = SK ? static_cast<int>(static_cast<long>(K / kBK) * (part + 1) / parts) - kt_first : K / kBK;
+  if (SK) {
+    A += static_cast<size_t>(kt_first) * 128;
+    W += static_cast<size_t>(kt_first) * (static_cast<size_t>(N) * 32u);
+  }
 
   // ---- per-lane byte offsets of the async copies inside k tile 0 ----
   constexpr int kAOps = St::kAOps;
@@ -228,6 +253,7 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
       meta_dst[p] = St::kABytes + St::kBBytes + idx * 256;
       meta_step[p] = kBlocks * meta_row_bytes;
     }
+    if (SK) meta_ptr[p] += static_cast<size_t>(kt_first) * meta_step[p];
   }
 
   const uint32_t lds0 = static_cast<uint32_t>(
@@ -546,12 +572,81 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   // (now unused) LDS ring, four row tiles at a time, and stores whole rows of its tile: 16 bytes per lane,
   // 64*NT contiguous bytes per row.
   block_barrier();  // nobody reads the ring any more
+  if (SK && parts > 1) {
+    // Partial tile of (split tile st, part): [wave][row tile][fragment][g][half][lane] pairs of floats -- a
+    // wave's store or load instruction covers 512 consecutive bytes.  The partial tiles and the counters are
+    // exchanged between workgroups on different XCDs, whose L2 caches do not see each other's lines.  So, per
+    // workgroup and not per wave (the cache operations act on the XCD's whole L2, and every invalidate throws
+    // away the operands the other workgroups of the XCD are working on): once all waves' stores have completed,
+    // ONE thread writes the L2's dirty lines back (release) and counts the workgroup in; in the workgroup that
+    // arrives last, ONE thread invalidates (acquire) before anybody reads the other parts.  The accesses
+    // themselves are device-scope atomic accesses, which bypass the compute unit's own cache.  (A workspace in
+    // uncached memory needs none of the cache operations; measured, that saves 1 us of 18 and is not used.)
+    constexpr int kTilePairs = kComputeWaves * RT * NT * 8 * 64;  // 8-byte pairs per partial tile
+    constexpr uint32_t kFlagOffset = kStages * St::kBytes - 64;   // behind the epilogue's staging area
+    const int st = tile - whole_tiles;
+    uint64_t* const tile_parts = reinterpret_cast<uint64_t*>(partials) + static_cast<size_t>(st) * parts * kTilePairs +
+                                 (wm * WN + wn) * (RT * NT * 8 * 64) + lane;
+    uint64_t* const mine = tile_parts + static_cast<size_t>(part) * kTilePairs;
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int g2 = 0; g2 < 8; ++g2) {
+          // (the elements are copied out first: a bit cast applied to a vector element directly was compiled
+          // into a read of element 0)
+          const float lo = acc[r][t][2 * g2], hi = acc[r][t][2 * g2 + 1];
+          const uint64_t v = static_cast<uint64_t>(__float_as_uint(lo)) | static_cast<uint64_t>(__float_as_uint(hi)) << 32;
+          __hip_atomic_store(mine + ((r * NT + t) * 8 + g2) * 64, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    wait_vmcnt<0>();  // this wave's stores have completed
+    block_barrier();  // every wave's have
+    if (tid == 0) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      const int arrived = __hip_atomic_fetch_add(&counters[st], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (arrived == parts - 1) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        // nobody else touches this counter any more in this launch: back to zero for the next one
+        __hip_atomic_store(&counters[st], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      lds_write_8(lds0 + kFlagOffset, 0, static_cast<uint32_t>(arrived), 0u);
+    }
+    block_barrier();
+    const int arrived = static_cast<int>(lds_read_16(lds0 + kFlagOffset).x);
+    if (arrived != parts - 1) return;  // somebody else finishes this tile
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[r][t][e] = 0.f;
+    constexpr int kPieces = RT * NT * 8;                   // pairs per lane
+    constexpr int kChunk = kPieces < 32 ? kPieces : 32;    // loaded at a time (registers)
+    for (int p = 0; p < parts; ++p) {  // fixed order, whoever arrived last: 0 + part 0 + part 1 + ...
+      const uint64_t* src = tile_parts + static_cast<size_t>(p) * kTilePairs;
+#pragma unroll
+      for (int x0 = 0; x0 < kPieces; x0 += kChunk) {
+        uint64_t v[kChunk];
+#pragma unroll
+        for (int x = 0; x < kChunk; ++x) {
+          v[x] = __hip_atomic_load(src + (x0 + x) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int x = 0; x < kChunk; ++x) {
+          const int rt_ = (x0 + x) / 8, g2 = (x0 + x) % 8;
+          acc[rt_ / NT][rt_ % NT][2 * g2] += __uint_as_float(static_cast<uint32_t>(v[x]));
+          acc[rt_ / NT][rt_ % NT][2 * g2 + 1] += __uint_as_float(static_cast<uint32_t>(v[x] >> 32));
+        }
+      }
+    }
+  }
   {
     constexpr int kRowBytes = 64 * NT + 16;        // padded: consecutive rows start 4 (NT=2: 36) banks apart
     constexpr int kPassTiles = (RT < 4) ? RT : 4;  // row tiles staged at a time
     constexpr int kChunks = 4 * NT;                // 16-byte chunks per row
     constexpr int kRowsPerStore = 64 / kChunks;
-    static_assert(kComputeWaves * 32 * kPassTiles * kRowBytes <= kStages * St::kBytes, "staging area does not fit");
+    static_assert(kComputeWaves * 32 * kPassTiles * kRowBytes <= kStages * St::kBytes - 64, "staging area does not fit");
     const uint32_t region = lds0 + (wm * WN + wn) * (32 * kPassTiles * kRowBytes);
     const int srow = lane / kChunks, chunk = lane % kChunks;
     const int col = nw0 + chunk * 8;
@@ -589,58 +684,76 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   }
 }
 
-template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW = false>
+template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW, bool SK>
 int launch_one(const blkq4_gemm_args* a) {
   constexpr int BM = 32 * RT * WM;
   constexpr int kBN = 32 * NT * WN;
+  const blkq4_tile_plan& t = a->tile;
   const int m_tiles = (a->m + BM - 1) / BM;
   const int n_tiles = (a->n + kBN - 1) / kBN;
-  const dim3 grid(static_cast<unsigned>(m_tiles) * n_tiles);
+  const int tiles = m_tiles * n_tiles;
+  if (a->launched_id != nullptr) *a->launched_id = tile_id(RT, NT, WM, WN, PW, SK);
+  if (a->dry_run) return 0;
+  int whole = tiles, split_tiles = 0, split_k = 1;
+  float* partials = nullptr;
+  int* counters = nullptr;
+  if (SK) {
+    // what the kernel assumes about the workspace, checked here: counters first, then the partial tiles
+    split_tiles = t.split_tiles;
+    split_k = t.split_k;
+    whole = tiles - split_tiles;
+    const size_t need = kCounterBytes + static_cast<size_t>(split_tiles) * split_k * BM * kBN * 4;
+    if (split_tiles < 1 || split_tiles > tiles || split_k < 2 || split_k > a->k / kBK ||
+        static_cast<size_t>(split_tiles) * sizeof(int) > kCounterBytes || a->workspace == nullptr ||
+        a->workspace_bytes < need || (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+    counters = static_cast<int*>(a->workspace);
+    partials = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + kCounterBytes);
+  }
+  const dim3 grid(static_cast<unsigned>(whole + split_tiles * split_k));
   // the launch's own status: a sticky error of an earlier, unrelated call stays where it is
-  return static_cast<int>(launch_status(gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW, ROW>, grid,
+  return static_cast<int>(launch_status(gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW, ROW, SK>, grid,
                                         dim3(64 * (WM * WN + PW)), 0, a->stream, static_cast<const uint8_t*>(a->a),
                                         static_cast<const uint8_t*>(a->packed_w),
                                         static_cast<const uint8_t*>(a->scales),
                                         static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c),
-                                        static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k, m_tiles));
+                                        static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k, m_tiles, whole,
+                                        split_tiles, split_k, partials, counters));
 }
 
+// The tile shapes that exist, (RT, NT, WM, WN, PW): what blkq4::choose() may ask for.  Those with whole rows
+// of 32 or 64 (one row tile only) have no split form and no form for blocks along N.
+#define BLKQ4_TILE_SHAPES(X) X(8, 2, 1, 4, 0) X(4, 2, 1, 4, 4) X(4, 1, 1, 4, 4) X(2, 1, 1, 4, 4)
+#define BLKQ4_TILE_SHAPES_ONE_ROW_TILE(X) X(1, 1, 1, 4, 4) X(1, 1, 1, 8, 0) X(2, 1, 1, 8, 0)
+
 template <int BS, bool HAS_ZP>
-int launch_rt(const blkq4_gemm_args* a) {
-  // Problems with at least one 256 x 256 tile per compute unit: four waves of 256 x 64 each, the
-  // fewest conversion instructions per MFMA (every register of a SIMD belongs to one wave, which
-  // leaves no room for producer waves).  Smaller ones: 128 x 256 tiles, four waves of 128 x 64 plus
-  // four producer waves.  Problems that 128 x 128 tiles cover in one round of workgroups take those
-  // (four waves of 128 x 32): twice the workgroups, each done in 0.6 of the time; and those that even
-  // 64 x 128 tiles cover in one round take these (four waves of 64 x 32; M = 256, K = N = 4096: 25.1 -> 20.9 us).
-  constexpr int kComputeUnits = 256;
-  const long tiles = static_cast<long>((a->m + 255) / 256) * ((a->n + 255) / 256);
-  const long small_tiles = static_cast<long>((a->m + 127) / 128) * ((a->n + 127) / 128);
-  const long smallest_tiles = static_cast<long>((a->m + 63) / 64) * ((a->n + 127) / 128);
-  if (!a->column_wise) {
-    // blocks along N (the streaming kernel takes the small row counts)
-    if (tiles >= kComputeUnits) return launch_one<BS, HAS_ZP, 8, 2, 1, 4, 0, true>(a);
-    if (smallest_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 2, 1, 1, 4, 4, true>(a);
-    if (small_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 4, 1, 1, 4, 4, true>(a);
-    return launch_one<BS, HAS_ZP, 4, 2, 1, 4, 4, true>(a);
+int launch_plan(const blkq4_gemm_args* a) {
+  const blkq4_tile_plan& t = a->tile;
+  const bool sk = t.split_k > 1;
+#define BLKQ4_TRY(RT_, NT_, WM_, WN_, PW_)                                                              \
+  if (t.rt == RT_ && t.nt == NT_ && t.wm == WM_ && t.wn == WN_ && t.pw == PW_) {                        \
+    if (a->column_wise) {                                                                               \
+      return sk ? launch_one<BS, HAS_ZP, RT_, NT_, WM_, WN_, PW_, false, true>(a)                       \
+                : launch_one<BS, HAS_ZP, RT_, NT_, WM_, WN_, PW_, false, false>(a);                     \
+    }                                                                                                   \
+    return sk ? launch_one<BS, HAS_ZP, RT_, NT_, WM_, WN_, PW_, true, true>(a)                          \
+              : launch_one<BS, HAS_ZP, RT_, NT_, WM_, WN_, PW_, true, false>(a);                        \
   }
-  // rows per workgroup: no more than the problem has
-  // (up to 64 rows: 128 columns with four waves and four producer waves when such tiles fill the chip in one
-  // round, else 256 columns with eight waves; M = 64, K = 4096, N = 28672: 34.7 against 26.3 us)
-  const bool one_round_of_128 = a->n / 128 >= 224 && a->n / 128 <= kComputeUnits;
-  if (a->m <= 32 && one_round_of_128) return launch_one<BS, HAS_ZP, 1, 1, 1, 4, 4>(a);
-  if (a->m <= 32) return launch_one<BS, HAS_ZP, 1, 1, 1, 8, 0>(a);
-  if (a->m <= 64 && one_round_of_128) return launch_one<BS, HAS_ZP, 2, 1, 1, 4, 4>(a);
-  if (a->m <= 64) return launch_one<BS, HAS_ZP, 2, 1, 1, 8, 0>(a);
-  if (tiles >= kComputeUnits) return launch_one<BS, HAS_ZP, 8, 2, 1, 4, 0>(a);
-  if (smallest_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 2, 1, 1, 4, 4>(a);
-  if (small_tiles <= kComputeUnits) return launch_one<BS, HAS_ZP, 4, 1, 1, 4, 4>(a);
-  return launch_one<BS, HAS_ZP, 4, 2, 1, 4, 4>(a);
+  BLKQ4_TILE_SHAPES(BLKQ4_TRY)
+#undef BLKQ4_TRY
+#define BLKQ4_TRY(RT_, NT_, WM_, WN_, PW_)                                                              \
+  if (t.rt == RT_ && t.nt == NT_ && t.wm == WM_ && t.wn == WN_ && t.pw == PW_ && a->column_wise && !sk) { \
+    return launch_one<BS, HAS_ZP, RT_, NT_, WM_, WN_, PW_, false, false>(a);                            \
+  }
+  BLKQ4_TILE_SHAPES_ONE_ROW_TILE(BLKQ4_TRY)
+#undef BLKQ4_TRY
+  return static_cast<int>(hipErrorInvalidValue);  // a shape that does not exist
 }
 
 template <int BS>
 int launch_bs(const blkq4_gemm_args* a) {
-  return a->zero_points ? launch_rt<BS, true>(a) : launch_rt<BS, false>(a);
+  return a->zero_points ? launch_plan<BS, true>(a) : launch_plan<BS, false>(a);
 }
 
 }  // namespace

@@ -35,6 +35,7 @@
 
 #include <stdint.h>
 
+#include "blkq4_choose.h"
 #include "blkq4_dequant.h"
 #include "blkq4_device.h"
 #include "blkq4_launch.h"
@@ -63,10 +64,6 @@ constexpr bool kBF = true;
 #else
 constexpr bool kBF = false;
 #endif
-
-// Where a wave finds its activation fragments.
-constexpr int kRowsWholeInLds = 1;   // all rows, all of K, staged once per workgroup
-constexpr int kRowsPerSlotInLds = 2; // 16 * MT rows x 128 k staged per slot, private to the wave
 
 template <int BS, int NT, int MT, int AM, bool ROW>
 struct Slot {
@@ -460,227 +457,103 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 #undef BLKQ4_LOAD_SLOT
 }
 
-// The kernel is bound by instruction issue as much as by the weight stream, so what matters is how
-// evenly the workgroups fill the 256 compute units: with T column tiles per workgroup the busiest
-// unit works through ceil(workgroups / 256) * T tiles.  Wider workgroups also re-read the activation
-// rows less often, which weighs more the more rows there are.
-constexpr size_t kMaxLdsBytes = 160 * 1024;
-constexpr int kStreamingMaxRows = 1024;
-constexpr int kComputeUnits = 256;
-constexpr int kPersistentFactor = 2;  // column groups per workgroup from which on workgroups walk
-
-
-void choose_shape(int m, int n, int k, int* nt, int* depth) {
-  const int tiles = n / 16;
-  // cost of fetching the activation rows relative to one tile's work: small while they are staged once per
-  // workgroup; when K is too long for that they are fetched again for every column group, 16 rows x 2 bytes
-  // against a tile's 16 columns x 1/2 byte per k
-  int rows = 1;
-  while (rows < m) rows *= 2;
-  const bool rows_fit = static_cast<size_t>(rows) * static_cast<size_t>(k) * 2 <= kMaxLdsBytes;
-  const float a_weight = !rows_fit ? static_cast<float>(rows) / 4.0f : (m > 4) ? 0.2f : 0.05f;
-  float best = 0.f;
-  *nt = 1;
-  for (int t = 1; t <= 3; ++t) {
-    const int wgs = (tiles + t - 1) / t;
-    const int rounds = (wgs + kComputeUnits - 1) / kComputeUnits;
-    const float cost = static_cast<float>(rounds) * (static_cast<float>(t) + a_weight);
-    if (t == 1 || cost < best) {
-      best = cost;
-      *nt = t;
-    }
-  }
-  // one tile per workgroup: 8 slices in flight while at most two workgroups share a unit, else 4
-  // (the deeper ring needs too many registers for more resident waves)
-  *depth = (*nt == 1 && tiles <= 2 * kComputeUnits) ? 8 : 4;
-}
-
 // Raises a kernel's dynamic-LDS limit, once per kernel instantiation and device.
 template <auto kKernel>
 hipError_t raise_lds_limit() {
   return raise_lds_limit_once(reinterpret_cast<const void*>(kKernel), kMaxLdsBytes, &lds_limit_flags<kKernel>());
 }
 
-// One kernel instantiation: raises its dynamic-LDS limit, then launches `row_groups` row groups of
-// 16 * MT rows each.
-template <int BS, bool HAS_ZP, bool ROW, int DEPTH, int NT, int MT, int kWaves, int AM, int kSplit = kWaves>
-int launch_kernel(const blkq4_gemm_args* a, int rows_log2, int row_groups = 1) {
+// One kernel instantiation with the launch geometry of the plan (blkq4_choose.h): raises its dynamic-LDS limit,
+// then launches.  What the kernel assumes about the plan is checked here.
+template <int BS, bool HAS_ZP, bool ROW, int DEPTH, int NT, int MT, int kWaves, int AM, int kSplit>
+int launch_kernel(const blkq4_gemm_args* a) {
+  const blkq4_streaming_plan& p = a->streaming;
   constexpr size_t kRedBytes = (kSplit == 1) ? 0 : static_cast<size_t>(kWaves) * NT * MT * 64 * 4 * 4;
   constexpr size_t kPerSlotBytes = static_cast<size_t>(kWaves) * DEPTH * 16 * MT * 256;
   static_assert(kRedBytes <= kMaxLdsBytes, "partial tiles do not fit in LDS");
   static_assert(AM != kRowsPerSlotInLds || kPerSlotBytes <= kMaxLdsBytes, "slots do not fit in LDS");
-  // the rows are copied 1 KiB at a time; the partial tiles of the reduction reuse their space
-  const size_t a_bytes = AM == kRowsWholeInLds ? ((((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023})
-                         : AM == kRowsPerSlotInLds ? kPerSlotBytes
-                                                   : 0;
+  const bool refill = p.refill != 0;
+  if (a->launched_id != nullptr) *a->launched_id = streaming_id(DEPTH, NT, MT, kWaves, AM, kSplit, refill);
+  if (a->dry_run) return 0;
+  const size_t a_bytes = AM == kRowsWholeInLds ? ((((static_cast<size_t>(a->k) * 2) << p.rows_log2) + 1023) & ~size_t{1023})
+                                               : kPerSlotBytes;
   constexpr int kGroupTiles = NT * (kWaves / kSplit);
   const int col_groups = (a->n / 16 + kGroupTiles - 1) / kGroupTiles;
-  int cg_stride = (col_groups + 31) / 32 * 32;  // one column group per workgroup
-  size_t lds_bytes = a_bytes > kRedBytes ? a_bytes : kRedBytes;
-  size_t red_offset = 0;
-  // Many more workgroups than the chip holds at once: a workgroup then walks over several column groups
-  // (cg, cg + cg_stride, ...) and requests the first slices of the next one while it finishes the current
-  // one, so only the first column group of a workgroup waits for its weights with nothing else to do.
-  // The partial tiles then get LDS of their own: the rows stay where they are for the next column group.
-  // (not the sixteen-wave kernel for blocks along N: its walking variant does not fit in 128 registers)
-  constexpr bool kMayWalk = !(ROW && kWaves == 16);
-  if (kMayWalk && a_bytes + kRedBytes <= kMaxLdsBytes) {
-    const int by_lds = static_cast<int>(kMaxLdsBytes / (a_bytes + kRedBytes));
-    const int by_waves = 32 / kWaves;
-    const int resident = kComputeUnits * (by_lds < by_waves ? by_lds : by_waves);
-    int stride = (resident / row_groups) / 32 * 32;
-    if (stride < 32) stride = 32;
-    if (cg_stride >= kPersistentFactor * stride) {
-      cg_stride = stride;
-      lds_bytes = a_bytes + kRedBytes;
-      red_offset = a_bytes;
-    }
+  if ((1 << p.rows_log2) * p.row_groups < a->m || (MT == 1 && (1 << p.rows_log2) > 16) || (MT == 2 && p.rows_log2 != 5) ||
+      p.row_groups < 1 || p.cg_stride < 32 || (p.cg_stride % 32) != 0 || p.lds_bytes > kMaxLdsBytes ||
+      p.red_offset + kRedBytes > p.lds_bytes || a_bytes > p.lds_bytes || (p.red_offset != 0 && p.red_offset < a_bytes) ||
+      (!refill && (p.cg_stride < col_groups || kSplit == 1)) ||
+      p.grid != static_cast<uint32_t>(p.cg_stride) * static_cast<uint32_t>(p.row_groups) ||
+      (kSplit == 1 && (reinterpret_cast<uintptr_t>(a->c) & 7u) != 0)) {
+    return static_cast<int>(hipErrorInvalidValue);
   }
-  const unsigned grid = static_cast<unsigned>(cg_stride) * static_cast<unsigned>(row_groups);
-  // workgroups walk over several column groups, or waves stream all of K by themselves
-  const bool refill = cg_stride < col_groups || kSplit == 1;
   auto launch = [&](auto* kernel, hipError_t attr) {
     if (attr != hipSuccess) return static_cast<int>(attr);
     // the launch's own status: a sticky error of an earlier, unrelated call stays where it is
-    return static_cast<int>(launch_status(kernel, dim3(grid), dim3(64 * kWaves), lds_bytes, a->stream,
+    return static_cast<int>(launch_status(kernel, dim3(p.grid), dim3(64 * kWaves), p.lds_bytes, a->stream,
                                           static_cast<const uint16_t*>(a->a), static_cast<const uint4*>(a->packed_w),
                                           static_cast<const uint16_t*>(a->scales),
                                           static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c),
-                                          static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k, rows_log2,
-                                          row_groups, cg_stride, static_cast<uint32_t>(red_offset)));
+                                          static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k, p.rows_log2,
+                                          p.row_groups, p.cg_stride, p.red_offset));
   };
   if (refill) {
-    constexpr auto kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, true, kSplit>;
-    return launch(kernel, raise_lds_limit<kernel>());
+    // (the sixteen-wave kernel for blocks along N has no walking variant: it does not fit in 128 registers)
+    if constexpr (ROW && kWaves == 16) {
+      return static_cast<int>(hipErrorInvalidValue);
+    } else {
+      constexpr auto kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, true, kSplit>;
+      return launch(kernel, raise_lds_limit<kernel>());
+    }
   }
   if constexpr (kSplit == 1) {
-    return static_cast<int>(hipErrorInvalidValue);  // not reached
+    return static_cast<int>(hipErrorInvalidValue);  // waves that do not split K exist in the walking form only
   } else {
     constexpr auto kernel = skinny_mfma_kernel<BS, HAS_ZP, DEPTH, NT, MT, kWaves, AM, ROW, false, kSplit>;
     return launch(kernel, raise_lds_limit<kernel>());
   }
 }
 
-// Slices that `waves` waves with rings of `depth` slices request for one column group: every wave asks for
-// whole rings, also when it has fewer slices left.
-int requested_slices(int k, int waves, int depth) {
-  const int slices = (k / 32 + 3) / 4;
-  int total = 0;
-  for (int w = 0; w < waves; ++w) {
-    const int mine = (slices - w + waves - 1) / waves;
-    total += (mine + depth - 1) / depth * depth;
-  }
-  return total;
-}
-
-// M <= 16, enough column tiles to give every wave the chip can hold one of its own, and rows small enough for
-// several workgroups per compute unit: the waves do not split K, each streams all of K for its own tile:
-// no sums across waves, no barriers, and a ring that stays full from the first slice to the last.
-template <int BS, bool HAS_ZP, bool ROW>
-bool launch_independent_waves(const blkq4_gemm_args* a, int* status) {
-  int rows_log2 = 0;
-  while ((1 << rows_log2) < a->m) ++rows_log2;
-  const size_t a_bytes = (((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023};
-  // measured break-even against workgroups that split K and walk (blocks along N gain more: their sixteen-wave
-  // kernel has no walking variant)
-  constexpr size_t kIndependentMaxRowBytes = (ROW ? 32 : 16) * 1024;
-  // (from 832 tiles on when K is no multiple of what the splitting waves' rings hold, which then ask for a
-  // fifth more slices than there are: K = 5120, N = 13824: 14.5 -> 12.7 us)
-  const int slices = (a->k / 32 + 3) / 4;
-  const bool rings_fit_k = 5 * requested_slices(a->k, 16, 2) < 6 * slices || 5 * requested_slices(a->k, 8, 4) < 6 * slices;
-  const int kIndependentMinTiles = ROW ? 896 : rings_fit_k ? 2000 : 832;
-  if (a->n / 16 < kIndependentMinTiles || a_bytes > kIndependentMaxRowBytes ||
-      (reinterpret_cast<uintptr_t>(a->c) & 7u) != 0) {
-    return false;
-  }
-  // four slices in flight per wave: with eight the kernel needs 90 registers and a SIMD holds five waves
-  // instead of seven, which costs more than the deeper ring gains (52 against 55 us at N = 128256)
-  *status = launch_kernel<BS, HAS_ZP, ROW, 4, 1, 1, 4, kRowsWholeInLds, 1>(a, rows_log2);
-  return true;
-}
-
-// M <= 16: one row tile; the waves of a workgroup split K.
-template <int BS, bool HAS_ZP, bool ROW, int DEPTH, int NT>
-int launch_waves(const blkq4_gemm_args* a) {
-  int rows_log2 = 0;
-  while ((1 << rows_log2) < a->m) ++rows_log2;
-  const size_t a_bytes = (((static_cast<size_t>(a->k) * 2) << rows_log2) + 1023) & ~size_t{1023};
-  // sixteen waves when there is enough K: each wave has less to convert after its last load has arrived,
-  // and more of that work overlaps the loads of the other waves.  With more workgroups than compute units,
-  // eight waves: smaller workgroups fill the units more evenly (M = 1, K = 4096, N = 14336: 11.4 -> 9.5 us),
-  // unless their rings would ask for many more slices than K has.
-  if (a->k >= 4096 && a_bytes <= kMaxLdsBytes) {
-    constexpr int kD8 = DEPTH > 4 ? 4 : DEPTH;
-    const int col_groups = (a->n / 16 + NT - 1) / NT;
-    if (!ROW && col_groups > kComputeUnits &&
-        20 * requested_slices(a->k, 8, kD8) <= 21 * requested_slices(a->k, 16, 2)) {
-      return launch_kernel<BS, HAS_ZP, ROW, kD8, NT, 1, 8, kRowsWholeInLds>(a, rows_log2);
-    }
-    return launch_kernel<BS, HAS_ZP, ROW, 2, NT, 1, 16, kRowsWholeInLds>(a, rows_log2);
-  }
-  if (a->k >= 1024) {
-    constexpr int kD = DEPTH > 4 ? 4 : DEPTH;
-    if (a_bytes <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, ROW, kD, NT, 1, 8, kRowsWholeInLds>(a, rows_log2);
-    return launch_kernel<BS, HAS_ZP, ROW, kD, NT, 1, 8, kRowsPerSlotInLds>(a, rows_log2);  // 8 * 4 * 4 KiB of rows
-  }
-  return launch_kernel<BS, HAS_ZP, ROW, DEPTH, NT, 1, 4, kRowsWholeInLds>(a, rows_log2);  // K < 1024: at most 32 KiB of rows
-}
-
-// M > 16: row groups of 32 rows (two row tiles share one conversion of the weights), NT column tiles per
-// workgroup, eight waves.
-template <int BS, bool HAS_ZP, bool ROW, int NT>
-int launch_rows(const blkq4_gemm_args* a, int row_groups) {
-  const size_t a_bytes = static_cast<size_t>(a->k) * 2 * 32;
-  if (a_bytes <= kMaxLdsBytes) return launch_kernel<BS, HAS_ZP, ROW, 2, NT, 2, 8, kRowsWholeInLds>(a, 5, row_groups);
-  return launch_kernel<BS, HAS_ZP, ROW, 2, NT, 2, 8, kRowsPerSlotInLds>(a, 5, row_groups);  // 8 * 2 * 8 KiB of rows
-}
+// The shapes that exist, (DEPTH, NT, MT, waves, AM, split): what blkq4::choose() may ask for.  Blocks along N:
+// those with one column tile per wave (28 registers of packed weights, scales and zero-points per slot and tile).
+#define BLKQ4_W kRowsWholeInLds
+#define BLKQ4_P kRowsPerSlotInLds
+#define BLKQ4_STREAMING_SHAPES(X)                                                                          \
+  /* row groups of 32 */                                                                                   \
+  X(2, 1, 2, 8, BLKQ4_W, 8) X(2, 2, 2, 8, BLKQ4_W, 8) X(2, 4, 2, 8, BLKQ4_W, 8)                            \
+  X(2, 1, 2, 8, BLKQ4_P, 8) X(2, 2, 2, 8, BLKQ4_P, 8) X(2, 4, 2, 8, BLKQ4_P, 8)                            \
+  /* waves with column tiles of their own */                                                               \
+  X(4, 1, 1, 4, BLKQ4_W, 1)                                                                                \
+  /* wide layers, rows staged per slice */                                                                 \
+  X(2, 4, 1, 4, BLKQ4_P, 4) X(2, 4, 1, 8, BLKQ4_P, 8)                                                      \
+  /* up to 16 rows, the waves split K */                                                                   \
+  X(4, 1, 1, 8, BLKQ4_W, 8) X(4, 2, 1, 8, BLKQ4_W, 8) X(4, 3, 1, 8, BLKQ4_W, 8)                            \
+  X(2, 1, 1, 16, BLKQ4_W, 16) X(2, 2, 1, 16, BLKQ4_W, 16) X(2, 3, 1, 16, BLKQ4_W, 16)                      \
+  X(4, 1, 1, 8, BLKQ4_P, 8) X(4, 2, 1, 8, BLKQ4_P, 8) X(4, 3, 1, 8, BLKQ4_P, 8)                            \
+  X(8, 1, 1, 4, BLKQ4_W, 4) X(4, 1, 1, 4, BLKQ4_W, 4) X(4, 2, 1, 4, BLKQ4_W, 4) X(4, 3, 1, 4, BLKQ4_W, 4)
 
 template <int BS, bool HAS_ZP, bool ROW>
-int launch_shape(const blkq4_gemm_args* a) {
-  if (a->m > 16) {
-    // Every workgroup fetches the 32 rows of its group for all of K, so wide workgroups (more column tiles)
-    // mean less activation traffic; but there should be a workgroup for most compute units (measured: four
-    // tiles per workgroup from 160 workgroups of four on, two from 160 of two on).
-    const int row_groups = (a->m + 31) / 32;
-    const long tiles = static_cast<long>(a->n / 16) * row_groups;
-    if (tiles >= 640) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 4>(a, row_groups);
-    if (tiles >= 320) return launch_rows<BS, HAS_ZP, ROW, ROW ? 1 : 2>(a, row_groups);
-    return launch_rows<BS, HAS_ZP, ROW, 1>(a, row_groups);
+int launch_plan(const blkq4_gemm_args* a) {
+  const blkq4_streaming_plan& p = a->streaming;
+#define BLKQ4_TRY(D_, NT_, MT_, W_, AM_, S_)                                                               \
+  if (p.depth == D_ && p.nt == NT_ && p.mt == MT_ && p.waves == W_ && p.am == AM_ && p.split == S_) {      \
+    if constexpr (ROW && NT_ > 1) {                                                                        \
+      return static_cast<int>(hipErrorInvalidValue);                                                       \
+    } else {                                                                                               \
+      return launch_kernel<BS, HAS_ZP, ROW, D_, NT_, MT_, W_, AM_, S_>(a);                                 \
+    }                                                                                                      \
   }
-  int status;
-  if (launch_independent_waves<BS, HAS_ZP, ROW>(a, &status)) return status;
-  if constexpr (!ROW) {
-    // Wide N and more than four rows, or K too long for the rows to stay in LDS: the rows are staged per slice,
-    // a workgroup takes four column tiles (the rows are fetched again for every column group) and a wave keeps
-    // two slices in flight, so that the slots are small enough for several workgroups per compute unit: eight
-    // waves from 832 column tiles on, four from 1536 on.  Measured against every other shape of workgroup:
-    // M = 16, K = 8192: N = 14336 24.3 -> 17.6 us, N = 28672 43.1 -> 34.1 us; rows that would fit (M = 16,
-    // K = 4096, N = 14336: 13.2 -> 11.1 us) gain less or nothing, never lose more than 3 %.
-    int rows_log2 = 0;
-    while ((1 << rows_log2) < a->m) ++rows_log2;
-    const bool rows_fit = ((static_cast<size_t>(a->k) * 2) << rows_log2) <= kMaxLdsBytes;
-    const int tiles = a->n / 16;
-    if ((!rows_fit || a->m > 4) && a->k >= 1024) {
-      if (tiles >= 1536) return launch_kernel<BS, HAS_ZP, ROW, 2, 4, 1, 4, kRowsPerSlotInLds>(a, rows_log2);
-      if (tiles >= 832) return launch_kernel<BS, HAS_ZP, ROW, 2, 4, 1, 8, kRowsPerSlotInLds>(a, rows_log2);
-    }
-  }
-  int nt, depth;
-  choose_shape(a->m, a->n, a->k, &nt, &depth);
-  if (ROW) {
-    // blocks along N: 28 registers of packed weights, scales and zero-points per slot and tile, so one tile
-    return (depth == 8) ? launch_waves<BS, HAS_ZP, ROW, 8, 1>(a) : launch_waves<BS, HAS_ZP, ROW, 4, 1>(a);
-  }
-  if (nt == 1 && depth == 8) return launch_waves<BS, HAS_ZP, ROW, 8, 1>(a);
-  if (nt == 1) return launch_waves<BS, HAS_ZP, ROW, 4, 1>(a);
-  if (nt == 2) return launch_waves<BS, HAS_ZP, ROW, 4, ROW ? 1 : 2>(a);
-  return launch_waves<BS, HAS_ZP, ROW, 4, ROW ? 1 : 3>(a);
+  BLKQ4_STREAMING_SHAPES(BLKQ4_TRY)
+#undef BLKQ4_TRY
+  return static_cast<int>(hipErrorInvalidValue);  // a shape that does not exist
 }
+#undef BLKQ4_W
+#undef BLKQ4_P
 
 template <int BS>
 int launch_skinny(const blkq4_gemm_args* a) {
-  if (a->column_wise) return a->zero_points ? launch_shape<BS, true, false>(a) : launch_shape<BS, false, false>(a);
-  return a->zero_points ? launch_shape<BS, true, true>(a) : launch_shape<BS, false, true>(a);
+  if (a->column_wise) return a->zero_points ? launch_plan<BS, true, false>(a) : launch_plan<BS, false, false>(a);
+  return a->zero_points ? launch_plan<BS, true, true>(a) : launch_plan<BS, false, true>(a);
 }
 
 }  // namespace

@@ -163,6 +163,28 @@ int blkq4_bf16_gemm_sm80(
   void* error_message);
 
 /**
+ * Which kernel a GEMM of this shape runs, without running it.  Host-only.  chosen_id receives the identity of the
+ * kernel the library's cost model picks for (m, n, k), launched_id the identity of the kernel instantiation its
+ * launcher maps that choice to -- the two are equal unless the library is broken -- and description (if not
+ * null, description_size bytes) a line of text such as "tile: 128 x 256, 4 + 4 waves, 258 tiles, the last 2 in
+ * 8 parts".  Any of the three may be null.
+ *
+ * No counterpart in the reference, whose choice is a single `m > 16` (src/blkq4_f16_gemm_sm80.cu:343): it exists
+ * so that a test can check, on a machine without a GPU, that the choice and the launchers agree for every shape,
+ * and so that a user can ask what a shape gets.
+ */
+int blkq4_gemm_plan_sm80(
+    int block_size,
+    bool column_wise_blocking,
+    bool bf16,
+    bool has_offsets,
+    int m, int n, int k,
+    uint64_t* chosen_id,
+    uint64_t* launched_id,
+    char* description, size_t description_size,
+    void* error_message);
+
+/**
  * Helpers for callers that cannot construct a C++ std::string (ctypes, cgo, JNI ...): create an
  * error-message object to pass as `error_message`, read it, destroy it.  Host-only; no counterpart
  * in the reference, whose callers are all C++.

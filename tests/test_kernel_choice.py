@@ -1,0 +1,80 @@
+"""The kernel choice (gemmlib_amd/csrc/blkq4_choose.h) and the launchers' dispatch agree, checked without a GPU
+through blkq4_gemm_plan_sm80: for every shape the identity of the kernel the cost model picks equals the identity
+of the kernel instantiation the launcher maps that choice to (a dry run: nothing is launched).
+
+The reference's own choice is `m > 16` between two kernels (src/blkq4_f16_gemm_sm80.cu:343,
+src/mickey/blk_q4/f16_gemm_sm80.h:63-72); the families below keep that much of it: GEMV and small batches stream
+the weights, prefill shapes run MFMA tiles."""
+
+import itertools
+
+import pytest
+
+MS = [1, 2, 4, 5, 8, 9, 16, 17, 24, 32, 33, 48, 64, 65, 96, 100, 128, 160, 200, 256, 300, 384, 512, 640, 768, 1000,
+      1024, 1025, 1536, 2048, 3000, 4096, 8192]
+NS = [32, 64, 256, 1024, 4096, 5120, 8192, 11008, 13824, 14336, 22016, 28672, 32000, 128256]
+KS = [64, 128, 512, 1024, 2048, 4096, 5120, 8192, 11008, 14336, 28672]
+
+
+def test_choice_equals_dispatch_over_a_sweep_of_shapes(capi):
+    checked = 0
+    kinds = set()
+    for col, bf16 in itertools.product((True, False), (False, True)):
+        for m, n, k in itertools.product(MS, NS, KS):
+            if not col and n % 64:
+                continue
+            chosen, launched, text = capi.gemm_plan(64, col, m, n, k, has_offsets=(m + n + k) % 3 != 0, bf16=bf16)
+            assert chosen == launched and chosen != 0, (col, bf16, m, n, k, hex(chosen), hex(launched), text)
+            kinds.add(chosen)
+            checked += 1
+    assert checked > 15000 and len(kinds) >= 25  # many different kernels were asked for, every one of them exists
+
+
+@pytest.mark.parametrize("bs", [16, 32, 64])
+def test_every_block_size_has_every_kernel(capi, bs):
+    for col in (True, False):
+        for m, n, k in [(1, 4096, 4096), (16, 11008, 4096), (16, 28672, 8192), (1, 128256, 4096), (64, 4096, 4096),
+                        (128, 4096, 4096), (256, 4096, 4096), (256, 4096, 11008), (768, 11008, 4096), (2048, 4096, 4096),
+                        (4096, 28672, 8192), (32, 28672, 8192), (64, 28672, 4096), (1280, 14336, 8192)]:
+            if not col and n % bs:
+                continue
+            chosen, launched, _ = capi.gemm_plan(bs, col, m, n, k)
+            assert chosen == launched
+
+
+def test_benchmark_configurations_get_the_expected_families(capi):
+    plans = {name: capi.gemm_plan(bs, True, m, n, k, has_offsets=zp)[2] for name, (m, k, n, bs, zp) in {
+        "C1": (64, 1024, 1024, 32, True), "C2": (1, 4096, 4096, 64, False), "C3": (16, 4096, 11008, 32, True),
+        "C4": (2048, 4096, 4096, 64, True), "C5": (4096, 8192, 28672, 16, True)}.items()}
+    assert plans["C2"].startswith("streaming: 16 waves splitting K")
+    assert plans["C3"].startswith("streaming:")
+    assert plans["C1"].startswith("streaming:")
+    assert plans["C4"].startswith("tile: 128 x 256, 4 + 4 waves, 256 tiles") and "parts" not in plans["C4"]
+    assert plans["C5"].startswith("tile: 256 x 256, 4 + 0 waves, 1792 tiles") and "parts" not in plans["C5"]
+
+
+def test_split_plans_are_well_formed(capi):
+    import re
+    seen = 0
+    for m, n, k in itertools.product([65, 100, 128, 200, 256, 300, 512, 768, 1280], [2048, 4096, 5120, 8192, 11008, 14336, 28672],
+                                     [1024, 4096, 5120, 8192, 11008, 14336, 28672]):
+        text = capi.gemm_plan(64, True, m, n, k)[2]
+        got = re.match(r"tile: (\d+) x (\d+), \d \+ \d waves, (\d+) tiles, the last (\d+) in (\d+) parts \(workspace (\d+) bytes\)", text)
+        if not got:
+            continue
+        seen += 1
+        bm, bn, tiles, split_tiles, parts, ws = map(int, got.groups())
+        assert tiles == -(-m // bm) * -(-n // bn)
+        assert split_tiles == (tiles % 256 or tiles) and 2 <= parts <= 4 and split_tiles * parts <= 256
+        assert (k // 64) // parts >= 4                                     # every part has at least 4 k tiles
+        assert ws == 16384 + split_tiles * parts * bm * bn * 4 <= 16384 + (32 << 20)
+    assert seen > 50
+
+
+def test_plan_rejects_what_the_gemm_rejects(capi):
+    for args, message in [((48, True, 4, 64, 64), "Unsupported block size: 48"), ((32, True, 0, 64, 64), "Empty problem size: 0x64x64"),
+                          ((32, True, 4, 64, 96), "Kernel execution failed: Error Invalid Problem"),
+                          ((64, False, 4, 96, 64), "Kernel execution failed: Error Invalid Problem")]:
+        with pytest.raises(capi.Blkq4Error) as e:
+            capi.gemm_plan(*args)
+        assert str(e.value) == message
