@@ -186,7 +186,7 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
                size_t a_size, void const* weights_ptr, size_t weights_size, void const* scales_ptr,
                size_t scales_size, void const* offsets_ptr, size_t offsets_size, void const* bias_ptr,
                size_t bias_size, void* output_ptr, size_t output_size, void* err_msg_ptr,
-               blkq4::Choice* plan_out = nullptr) {
+               bool static_workspace = false) {
   auto* err = static_cast<std::string*>(err_msg_ptr);
   if (!supported_block_size(block_size)) {
     set_error(err, "Unsupported block size: " + std::to_string(block_size));
@@ -285,18 +285,27 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
   // library's own for this stream; when there is none to be had (out of memory, too many streams), the plan is
   // made again without one.
   blkq4::Choice choice = blkq4::choose(column_wise_blocking, m, n, k, blkq4_dev_workspace_capacity());
-  if (plan_out != nullptr) {
-    *plan_out = choice;
-    return 0;
-  }
   if (choice.family == blkq4::kFamilyTile && choice.t.split_k > 1) {
     void* workspace = nullptr;
-    if (int code = blkq4_dev_workspace(stream, &workspace)) return device_failure(code, err);
-    if (workspace == nullptr) {
-      choice = blkq4::choose(column_wise_blocking, m, n, k, 0);
-    } else {
+    if (static_workspace) {
+      // the allocation-free entry point: the same plan, the workspace that lives in the library's device image
+      if (choice.t.workspace_bytes > blkq4_dev_static_workspace_capacity()) {
+        set_error(err, "Workspace of " + std::to_string(choice.t.workspace_bytes) +
+                           " bytes needed, the allocation-free entry point holds " +
+                           std::to_string(blkq4_dev_static_workspace_capacity()));
+        return -1;
+      }
+      if (int code = blkq4_dev_static_workspace(&workspace)) return device_failure(code, err);
       args.workspace = workspace;
-      args.workspace_bytes = blkq4_dev_workspace_capacity();
+      args.workspace_bytes = blkq4_dev_static_workspace_capacity();
+    } else {
+      if (int code = blkq4_dev_workspace(stream, &workspace)) return device_failure(code, err);
+      if (workspace == nullptr) {
+        choice = blkq4::choose(column_wise_blocking, m, n, k, 0);
+      } else {
+        args.workspace = workspace;
+        args.workspace_bytes = blkq4_dev_workspace_capacity();
+      }
     }
   }
   args.streaming = choice.s;
@@ -349,6 +358,19 @@ extern "C" BLKQ4_EXPORT int blkq4_bf16_gemm_sm80(int block_size, bool column_wis
   return gemm_entry(true, block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr,
                     weights_size, scales_ptr, scales_size, offsets_ptr, offsets_size, bias_ptr, bias_size,
                     output_ptr, output_size, err_msg_ptr);
+}
+
+// blkq4_fp16_gemm_sm80 for callers that must not allocate: a split tile kernel's workspace is the buffer inside
+// the library's device image, never the library's own per-stream buffer (which is allocated on first use)
+extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_noalloc_sm80(int block_size, bool column_wise_blocking, int m, int n,
+                                                         int k, void* stream, void const* act_ptr, size_t a_size,
+                                                         void const* weights_ptr, size_t weights_size,
+                                                         void const* scales_ptr, size_t scales_size,
+                                                         void const* offsets_ptr, size_t offsets_size,
+                                                         void* output_ptr, size_t output_size, void* err_msg_ptr) {
+  return gemm_entry(false, block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
+                    scales_ptr, scales_size, offsets_ptr, offsets_size, nullptr, 0, output_ptr, output_size,
+                    err_msg_ptr, /*static_workspace=*/true);
 }
 
 // Which kernel a GEMM of this shape runs, without running it: the identity of the kernel blkq4::choose() picks

@@ -110,6 +110,10 @@ const char* blkq4_dev_error_string(int code);
  * made (out of memory, or too many streams have one). */
 size_t blkq4_dev_workspace_capacity(void);
 int blkq4_dev_workspace(void* stream, void** ptr);
+/* The workspace inside the library's device image (nothing is ever allocated): one per device, shared by every
+ * stream of that device. */
+size_t blkq4_dev_static_workspace_capacity(void);
+int blkq4_dev_static_workspace(void** ptr);
 
 #ifdef __cplusplus
 }

@@ -7,6 +7,11 @@
 //     it, as tensor libraries do for their own allocations during capture).  A recorded call keeps using the
 //     buffer of the stream it was recorded on, whatever stream the graph is launched on later.
 //
+//   blkq4_dev_static_workspace: a buffer inside the library's device image, for callers that must not allocate
+//     (code recorded into a graph by a harness that forbids it, tight serving loops).  Nothing is ever allocated;
+//     every GPU the library runs on holds its copy until the process ends.  One per device, shared by all of its
+//     streams: calls that overlap on one device race.  Its counters are zero when the image is loaded.
+//
 // The kernels leave the arrival counters at zero (the workgroup that arrives last clears its tile's counter), so
 // they are cleared once, when the buffer is allocated, by a small kernel on a stream of the allocation's own.
 
@@ -24,6 +29,13 @@ namespace {
 
 constexpr size_t kPoolBytes = blkq4::kCounterBytes + (size_t{32} << 20);
 constexpr int kMaxSlots = 16;  // streams with a buffer of their own; later ones run unsplit kernels
+constexpr size_t kStaticBytes = blkq4::kCounterBytes + (size_t{16} << 20);
+constexpr int kMaxDevices = 64;
+
+// Host code never uses this name as an address (it is a host-side stand-in for the symbol): it asks
+// hipGetSymbolAddress for the array's device address, once per device, and works with that.
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+void* g_static_ptr[kMaxDevices];  // each GPU holds its own copy of the array at its own address
 
 __global__ void clear_counters(int* counters) {
   for (unsigned i = threadIdx.x; i < blkq4::kCounterBytes / sizeof(int); i += blockDim.x) counters[i] = 0;
@@ -80,5 +92,24 @@ extern "C" int blkq4_dev_workspace(void* stream_ptr, void** ptr) {
   if (e != hipSuccess) return static_cast<int>(e);
   g_slots[g_slot_count++] = Slot{device, stream, p};
   *ptr = p;
+  return 0;
+}
+
+extern "C" size_t blkq4_dev_static_workspace_capacity(void) { return kStaticBytes; }
+
+extern "C" int blkq4_dev_static_workspace(void** ptr) {
+  *ptr = nullptr;
+  int device = 0;
+  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return static_cast<int>(e);
+  if (device < 0 || device >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (g_static_ptr[device] == nullptr) {
+    // set-up, once per device, with that device current
+    void* p = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)); e != hipSuccess) return static_cast<int>(e);
+    if (p == nullptr || (reinterpret_cast<uintptr_t>(p) & 255u) != 0) return static_cast<int>(hipErrorInvalidSymbol);
+    g_static_ptr[device] = p;
+  }
+  *ptr = g_static_ptr[device];
   return 0;
 }

@@ -163,6 +163,31 @@ int blkq4_bf16_gemm_sm80(
   void* error_message);
 
 /**
+ * blkq4_fp16_gemm_sm80 for callers that cannot allocate device memory: code recorded into a graph by a harness
+ * that forbids allocation, tight serving loops.  Same arguments, checks, messages, kernels and result bits as
+ * blkq4_fp16_gemm_sm80.  The difference: when the chosen kernel splits tiles over K and needs a workspace for the
+ * fp32 partial tiles, that workspace is a buffer inside the library's device image (16 MiB + 16 KiB per GPU, held
+ * until the process ends) instead of the per-stream buffer blkq4_fp16_gemm_sm80 allocates on first use.  No
+ * hipMalloc, hipFree or other allocating call is made.  A shape whose plan needs more than the buffer holds is
+ * rejected with "Workspace of N bytes needed, the allocation-free entry point holds M" (-1); blkq4_fp16_gemm_sm80
+ * takes such a shape.  All streams of a GPU share the one buffer: calls that overlap on one GPU race, so issue
+ * them on one stream or order them yourself.
+ *
+ * No counterpart in the reference (whose GEMM needs no workspace): it is for the callers that cannot allocate.
+ */
+int blkq4_fp16_gemm_noalloc_sm80(
+  int block_size,
+  bool column_wise_blocking,
+  int m, int n, int k,
+  void* stream,
+  void const* act_ptr, size_t a_size,
+  void const* weights_ptr, size_t weights_size,
+  void const* scales_ptr, size_t scales_size,
+  void const* offsets_ptr, size_t offsets_size,
+  void* output_ptr, size_t output_size,
+  void* error_message);
+
+/**
  * Which kernel a GEMM of this shape runs, without running it.  Host-only.  chosen_id receives the identity of the
  * kernel the library's cost model picks for (m, n, k), launched_id the identity of the kernel instantiation its
  * launcher maps that choice to -- the two are equal unless the library is broken -- and description (if not
