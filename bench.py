@@ -386,6 +386,46 @@ def bench_copy(torch, capi, device, steps, warmup):
     }
 
 
+GEMV_FORM_SHAPES = [(1, 4096, 4096, 64, False), (1, 4096, 4096, 64, True), (2, 4096, 4096, 64, False), (4, 4096, 4096, 64, False),
+                    (1, 2048, 2048, 64, False), (1, 2048, 8192, 64, False), (1, 4096, 11008, 32, True), (1, 8192, 4096, 64, False),
+                    (1, 11008, 4096, 64, False), (1, 14336, 4096, 64, False), (1, 8192, 8192, 64, False), (1, 8192, 28672, 64, False),
+                    (1, 4096, 128256, 64, False), (4, 4096, 14336, 64, True)]
+
+
+def bench_gemv_forms(torch, capi, device, shapes, steps):
+    """The two forms of the GEMV on the same data in the same process: the one blkq4_fp16_gemm_sm80 picks (MFMA:
+    every wave converts its weights and feeds v_mfma_f32_16x16x32_f16) and blkq4_fp16_gemv_valu_sm80 (no MFMA:
+    per-lane fp32 partial sums with v_dot2_f32_f16, lane exchanges across K).  shapes: (M, K, N, block size,
+    zero-points).  Weight sets rotate over twice the Infinity Cache."""
+    rows = []
+    for m, k, n, bs, zp in shapes:
+        per_set = k * n // 2 + 2 * k * n // bs + (k * n // bs if zp else 0)
+        copies = min(64, 2 * INFINITY_CACHE_BYTES // per_set + 1)
+        g = torch.Generator(device=device).manual_seed(7)
+        a = torch.randn(m, k, generator=g, device=device).to(torch.float16)
+        w_elems, meta = capi.quant_size(bs, True, k, n)
+        sets = []
+        for _ in range(copies):
+            w = (torch.randn(n, k, generator=g, device=device) * 0.02).to(torch.float16)
+            q_w = torch.empty(w_elems, dtype=torch.uint8, device=device)
+            q_s = torch.empty(meta, dtype=torch.float16, device=device)
+            q_z = torch.empty(meta, dtype=torch.uint8, device=device) if zp else None
+            capi.quant(bs, True, w, q_w, q_s, q_z)
+            sets.append((q_w, q_s, q_z))
+            del w
+        out = torch.empty(m, n, dtype=torch.float16, device=device)
+        n_launch = copies * ((max(steps, copies) + copies - 1) // copies)
+        row = {"shape": f"M={m} K={k} N={n} bs{bs} {'asym' if zp else 'sym'}", "weight_sets": copies}
+        for key, valu in (("mfma_us", False), ("valu_us", True)):
+            launches = [(lambda s=s: capi.gemm(bs, True, m, n, k, a, s[0], s[1], s[2], out, valu=valu)) for s in sets]
+            _, evt, _ = timed_region(torch, launches, n_launch, 5, settle_seconds=0.2)
+            row[key] = round(evt / n_launch * 1e6, 3)
+        rows.append(row)
+        del sets
+        torch.cuda.empty_cache()
+    return rows
+
+
 def bench_context(torch, capi, device, head_problem, steps, warmup):
     """Figures the headline numbers are read against, measured in the same run:
     * what a graph node costs when its kernel does nothing, and what a kernel costs that issues the GEMV's
@@ -432,6 +472,7 @@ def bench_context(torch, capi, device, head_problem, steps, warmup):
         wall, evt, _ = timed_region(torch, launches, floor_launches, warmup)
         out["c2_requests_only_us" if with_scales else "c2_weight_requests_only_us"] = round(evt / floor_launches * 1e6, 3)
     del ws, ss
+    out["gemv_forms_c2_shape"] = bench_gemv_forms(torch, capi, device, [(1, 4096, 4096, 64, False)], steps)[0]
     if head_problem is not None:
         a, sets, c, w_host = head_problem
         m, k, n, bs, has_offsets, _ = CONFIGS["C4"]
@@ -462,6 +503,8 @@ def main(argv=None) -> int:
     ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r,C2r,M128,M256,M512,M768N11K,M256K11K,V128K,B16,C4b,C2b")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-context", action="store_true", help="skip the floors and the library comparison")
+    ap.add_argument("--gemv-forms", action="store_true",
+                    help="only the A/B of the two forms of the GEMV (MFMA / no MFMA) over a list of shapes")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -476,6 +519,9 @@ def main(argv=None) -> int:
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    if args.gemv_forms:
+        print(json.dumps({"gemv_forms": bench_gemv_forms(torch, capi, device, GEMV_FORM_SHAPES, max(args.steps, 100))}))
+        return 0
     wanted = [c.strip() for c in args.configs.split(",") if c.strip()]
     with_cpu = not args.no_cpu
     results = {}

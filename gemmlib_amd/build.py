@@ -29,7 +29,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libms_blkq4gemm.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 HIP_SOURCES = ["blkq4_prepack.hip", "blkq4_skinny.hip", "blkq4_skinny_bf16.hip", "blkq4_gemm.hip", "blkq4_gemm_bf16.hip",
-               "blkq4_workspace.hip"]
+               "blkq4_workspace.hip", "blkq4_gemv.hip"]
 HOST_SOURCES = ["blkq4_api.cpp"]
 
 # -ffp-contract=off: every fused multiply-add the quantizer needs is written as an explicit fmaf.

@@ -24,6 +24,7 @@ EXPORTED_SYMBOLS = (
     "blkq4_bf16_gemm_sm80",
     "blkq4_gemm_plan_sm80",
     "blkq4_fp16_gemm_noalloc_sm80",
+    "blkq4_fp16_gemv_valu_sm80",
     "blkq4_error_message_create",
     "blkq4_error_message_cstr",
     "blkq4_error_message_destroy",
@@ -56,6 +57,8 @@ def load() -> ctypes.CDLL:
     L.blkq4_fp16_gemm_sm80.restype = i
     L.blkq4_fp16_gemm_noalloc_sm80.argtypes = L.blkq4_fp16_gemm_sm80.argtypes
     L.blkq4_fp16_gemm_noalloc_sm80.restype = i
+    L.blkq4_fp16_gemv_valu_sm80.argtypes = L.blkq4_fp16_gemm_sm80.argtypes
+    L.blkq4_fp16_gemv_valu_sm80.restype = i
     L.blkq4_fp16_gemm_bias_sm80.argtypes = [i, b, i, i, i, vp, vp, sz, vp, sz, vp, sz, vp, sz, vp, sz, vp, sz, vp]
     L.blkq4_fp16_gemm_bias_sm80.restype = i
     L.blkq4_fp16_quant_sm80.argtypes = [i, b, i, i, i, vp, vp, sz, vp, sz, vp, sz, vp, sz, vp]
@@ -157,14 +160,16 @@ def quant(block_size: int, column_wise: bool, weights_nk, q_weights, q_scales, q
 
 
 def gemm(block_size: int, column_wise: bool, m: int, n: int, k: int, a, q_weights, q_scales, q_zp, out,
-         stream=None, bias=None, bf16=False, noalloc=False):
+         stream=None, bias=None, bf16=False, noalloc=False, valu=False):
     """``blkq4_fp16_gemm_sm80`` on device tensors; with ``bias`` (fp16 ``[n]``) ``blkq4_fp16_gemm_bias_sm80``;
-    ``bf16=True``: ``blkq4_bf16_gemm_sm80`` (bias optional); ``noalloc=True``: ``blkq4_fp16_gemm_noalloc_sm80``."""
+    ``bf16=True``: ``blkq4_bf16_gemm_sm80`` (bias optional); ``noalloc=True``: ``blkq4_fp16_gemm_noalloc_sm80``;
+    ``valu=True``: ``blkq4_fp16_gemv_valu_sm80``."""
     L = load()
     err = _ErrMsg(L)
-    if noalloc:
+    if noalloc or valu:
         assert bias is None and not bf16
-        rc = L.blkq4_fp16_gemm_noalloc_sm80(block_size, column_wise, m, n, k, _stream_ptr(stream), _ptr(a), _nbytes(a),
+        entry = L.blkq4_fp16_gemv_valu_sm80 if valu else L.blkq4_fp16_gemm_noalloc_sm80
+        rc = entry(block_size, column_wise, m, n, k, _stream_ptr(stream), _ptr(a), _nbytes(a),
                                             _ptr(q_weights), _nbytes(q_weights), _ptr(q_scales), _nbytes(q_scales),
                                             _ptr(q_zp), _nbytes(q_zp), _ptr(out), _nbytes(out), err.h)
     elif bf16:

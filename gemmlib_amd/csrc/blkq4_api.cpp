@@ -186,7 +186,7 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
                size_t a_size, void const* weights_ptr, size_t weights_size, void const* scales_ptr,
                size_t scales_size, void const* offsets_ptr, size_t offsets_size, void const* bias_ptr,
                size_t bias_size, void* output_ptr, size_t output_size, void* err_msg_ptr,
-               bool static_workspace = false) {
+               bool static_workspace = false, bool valu_gemv = false) {
   auto* err = static_cast<std::string*>(err_msg_ptr);
   if (!supported_block_size(block_size)) {
     set_error(err, "Unsupported block size: " + std::to_string(block_size));
@@ -284,6 +284,15 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
   // src/blkq4_f16_gemm_sm80.cu:343, f16_gemm_sm80.h:63-72).  A split tile kernel needs a workspace: the
   // library's own for this stream; when there is none to be had (out of memory, too many streams), the plan is
   // made again without one.
+  if (valu_gemv) {
+    // the GEMV kernel without MFMA, asked for by name
+    if (m > 4 || !column_wise_blocking || bf16 || (m == 3 ? 4 : m) * K * 2 > 150 * 1024) {
+      set_error(err, "The GEMV without matrix instructions takes fp16, 1 to 4 rows of at most 150 KiB together and blocks along K");
+      return -1;
+    }
+    if (int code = blkq4_dev_gemv_dot(&args)) return device_failure(code, err);
+    return 0;
+  }
   blkq4::Choice choice = blkq4::choose(column_wise_blocking, m, n, k, blkq4_dev_workspace_capacity());
   if (choice.family == blkq4::kFamilyTile && choice.t.split_k > 1) {
     void* workspace = nullptr;
@@ -371,6 +380,20 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_noalloc_sm80(int block_size, bool co
   return gemm_entry(false, block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
                     scales_ptr, scales_size, offsets_ptr, offsets_size, nullptr, 0, output_ptr, output_size,
                     err_msg_ptr, /*static_workspace=*/true);
+}
+
+// blkq4_fp16_gemm_sm80 for 1 to 4 rows, computed by the kernel that uses no matrix instructions (per-lane fp32
+// partial sums, v_dot2_f32_f16, lane exchanges across K): the alternative form of the GEMV, kept callable by name
+// so that it can be measured against the form blkq4_fp16_gemm_sm80 picks
+extern "C" BLKQ4_EXPORT int blkq4_fp16_gemv_valu_sm80(int block_size, bool column_wise_blocking, int m, int n, int k,
+                                                      void* stream, void const* act_ptr, size_t a_size,
+                                                      void const* weights_ptr, size_t weights_size,
+                                                      void const* scales_ptr, size_t scales_size,
+                                                      void const* offsets_ptr, size_t offsets_size,
+                                                      void* output_ptr, size_t output_size, void* err_msg_ptr) {
+  return gemm_entry(false, block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
+                    scales_ptr, scales_size, offsets_ptr, offsets_size, nullptr, 0, output_ptr, output_size,
+                    err_msg_ptr, /*static_workspace=*/false, /*valu_gemv=*/true);
 }
 
 // Which kernel a GEMM of this shape runs, without running it: the identity of the kernel blkq4::choose() picks

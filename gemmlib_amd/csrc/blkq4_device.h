@@ -102,6 +102,7 @@ int blkq4_dev_gemm(const blkq4_gemm_args* args);   /* MFMA tile kernel, every m 
 int blkq4_dev_skinny(const blkq4_gemm_args* args); /* weight-streaming kernel, 1 <= m <= 1024 */
 int blkq4_dev_gemm_bf16(const blkq4_gemm_args* args);   /* the tile kernel with bf16 a, scales, c and bias */
 int blkq4_dev_skinny_bf16(const blkq4_gemm_args* args); /* the same with bf16 a, scales, c and bias */
+int blkq4_dev_gemv_dot(const blkq4_gemm_args* args);    /* fp16 GEMV on the vector ALU (no MFMA): 1 <= m <= 4, blocks along K */
 int blkq4_dev_repack(const blkq4_repack_args* args);
 const char* blkq4_dev_error_string(int code);
 

@@ -188,6 +188,28 @@ int blkq4_fp16_gemm_noalloc_sm80(
   void* error_message);
 
 /**
+ * The GEMV (1 <= m <= 4, fp16, column_wise_blocking = true) computed without matrix instructions: per-lane fp32
+ * partial sums over K with v_dot2_f32_f16, summed across the wave by lane exchanges and across the workgroup's
+ * waves through LDS.  Same arguments, checks and messages as blkq4_fp16_gemm_sm80, same dequantized weights, fp32
+ * accumulation and single rounding of the output; other shapes are rejected (-1).
+ *
+ * No counterpart in the reference (whose small-M kernel, src/mickey/blk_q4/f16_gemm_sm80.h:63-72, uses tensor
+ * cores too).  blkq4_fp16_gemm_sm80 picks between this form and the MFMA form by shape; this entry point runs this
+ * form whatever the shape, so that the two can be measured against each other.
+ */
+int blkq4_fp16_gemv_valu_sm80(
+  int block_size,
+  bool column_wise_blocking,
+  int m, int n, int k,
+  void* stream,
+  void const* act_ptr, size_t a_size,
+  void const* weights_ptr, size_t weights_size,
+  void const* scales_ptr, size_t scales_size,
+  void const* offsets_ptr, size_t offsets_size,
+  void* output_ptr, size_t output_size,
+  void* error_message);
+
+/**
  * Which kernel a GEMM of this shape runs, without running it.  Host-only.  chosen_id receives the identity of the
  * kernel the library's cost model picks for (m, n, k), launched_id the identity of the kernel instantiation its
  * launcher maps that choice to -- the two are equal unless the library is broken -- and description (if not
