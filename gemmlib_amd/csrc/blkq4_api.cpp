@@ -180,6 +180,13 @@ extern "C" BLKQ4_EXPORT int blkq4_bf16_quant_sm80(int block_size, bool column_wi
 
 namespace {
 
+int launch_choice(const blkq4::Choice& choice, bool bf16, const blkq4_gemm_args* args) {
+  if (choice.family == blkq4::kFamilyValuGemv) return blkq4_dev_gemv_dot(args);
+  const bool streaming = choice.family == blkq4::kFamilyStreaming;
+  return bf16 ? (streaming ? blkq4_dev_skinny_bf16(args) : blkq4_dev_gemm_bf16(args))
+              : (streaming ? blkq4_dev_skinny(args) : blkq4_dev_gemm(args));
+}
+
 // reference: src/blkq4_f16_gemm_sm80.cu:319-429 and :38-153 (blkq4_gemm_sm80_T); bias_ptr == nullptr or
 // bias_size == 0: no bias
 int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int n, int k, void* stream, void const* act_ptr,
@@ -293,7 +300,7 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
     if (int code = blkq4_dev_gemv_dot(&args)) return device_failure(code, err);
     return 0;
   }
-  blkq4::Choice choice = blkq4::choose(column_wise_blocking, m, n, k, blkq4_dev_workspace_capacity());
+  blkq4::Choice choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, blkq4_dev_workspace_capacity());
   if (choice.family == blkq4::kFamilyTile && choice.t.split_k > 1) {
     void* workspace = nullptr;
     if (static_workspace) {
@@ -310,7 +317,7 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
     } else {
       if (int code = blkq4_dev_workspace(stream, &workspace)) return device_failure(code, err);
       if (workspace == nullptr) {
-        choice = blkq4::choose(column_wise_blocking, m, n, k, 0);
+        choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, 0);
       } else {
         args.workspace = workspace;
         args.workspace_bytes = blkq4_dev_workspace_capacity();
@@ -319,10 +326,7 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
   }
   args.streaming = choice.s;
   args.tile = choice.t;
-  const bool streaming = choice.family == blkq4::kFamilyStreaming;
-  const int code = bf16 ? (streaming ? blkq4_dev_skinny_bf16(&args) : blkq4_dev_gemm_bf16(&args))
-                        : (streaming ? blkq4_dev_skinny(&args) : blkq4_dev_gemm(&args));
-  if (code) return device_failure(code, err);
+  if (int code = launch_choice(choice, bf16, &args)) return device_failure(code, err);
   return 0;
 }
 
@@ -417,7 +421,7 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
     set_error(err, "Kernel execution failed: Error Invalid Problem");
     return -1;
   }
-  const blkq4::Choice choice = blkq4::choose(column_wise_blocking, m, n, k, blkq4_dev_workspace_capacity());
+  const blkq4::Choice choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, blkq4_dev_workspace_capacity());
   blkq4_gemm_args args{};
   args.block_size = block_size;
   args.column_wise = column_wise_blocking ? 1 : 0;
@@ -435,14 +439,15 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
   uint64_t launched = 0;
   args.launched_id = &launched;
   const bool streaming = choice.family == blkq4::kFamilyStreaming;
-  const int code = bf16 ? (streaming ? blkq4_dev_skinny_bf16(&args) : blkq4_dev_gemm_bf16(&args))
-                        : (streaming ? blkq4_dev_skinny(&args) : blkq4_dev_gemm(&args));
-  if (code) return device_failure(code, err);
+  if (int code = launch_choice(choice, bf16, &args)) return device_failure(code, err);
   if (chosen_id != nullptr) *chosen_id = blkq4::choice_id(choice);
   if (launched_id != nullptr) *launched_id = launched;
   if (description != nullptr && description_size > 0) {
     std::string text;
-    if (streaming) {
+    if (choice.family == blkq4::kFamilyValuGemv) {
+      text = "gemv without MFMA: " + std::to_string(choice.valu_waves) + " waves splitting K, 16 columns x " +
+             std::to_string(choice.valu_rows) + " row(s), " + std::to_string(n / 16) + " workgroups";
+    } else if (streaming) {
       const auto& p = choice.s;
       text = "streaming: " + std::to_string(p.waves) + " waves" + (p.split == 1 ? " with column tiles of their own" : " splitting K") +
              ", " + std::to_string(p.nt) + " column tile(s) x " + std::to_string(16 * p.mt) + " rows, " +

@@ -26,6 +26,7 @@ constexpr int kRowsPerSlotInLds = 2;  // 16 * MT rows x 128 k staged per slot, p
 
 constexpr int kFamilyStreaming = 0;  // weight-streaming kernel (blkq4_skinny.hip)
 constexpr int kFamilyTile = 1;       // MFMA tile kernel (blkq4_gemm.hip)
+constexpr int kFamilyValuGemv = 2;   // GEMV without MFMA (blkq4_gemv.hip)
 
 using StreamingShape = blkq4_streaming_plan;  // see blkq4_device.h
 using TileShape = blkq4_tile_plan;
@@ -34,6 +35,7 @@ struct Choice {
   int family;
   StreamingShape s;
   TileShape t;
+  int valu_rows, valu_waves;  // kFamilyValuGemv
 };
 
 // A kernel's identity as one number: what choose() picked and what a launcher started can be compared.
@@ -47,7 +49,18 @@ inline uint64_t tile_id(int rt, int nt, int wm, int wn, int pw, bool split) {
          static_cast<uint64_t>(wm) << 24 | static_cast<uint64_t>(wn) << 16 | static_cast<uint64_t>(pw) << 8 |
          (split ? 1u : 0u);
 }
+// the GEMV without MFMA: rows kept (1, 2 or 4) and waves of a workgroup
+inline int valu_gemv_rows(int m) { return m == 1 ? 1 : m == 2 ? 2 : 4; }
+inline int valu_gemv_waves(int k) {
+  // sixteen waves when every one of them gets at least two 128-deep slices, else eight, else four
+  const int slices = (k / 32 + 3) / 4;
+  return slices >= 32 ? 16 : slices >= 16 ? 8 : 4;
+}
+inline uint64_t valu_gemv_id(int rows, int waves) {
+  return 3ull << 60 | static_cast<uint64_t>(rows) << 8 | static_cast<uint64_t>(waves);
+}
 inline uint64_t choice_id(const Choice& c) {
+  if (c.family == kFamilyValuGemv) return valu_gemv_id(c.valu_rows, c.valu_waves);
   return c.family == kFamilyStreaming
              ? streaming_id(c.s.depth, c.s.nt, c.s.mt, c.s.waves, c.s.am, c.s.split, c.s.refill != 0)
              : tile_id(c.t.rt, c.t.nt, c.t.wm, c.t.wn, c.t.pw, c.t.split_k > 1);
@@ -382,8 +395,18 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
 
 // The whole decision.  workspace_capacity: bytes of workspace the caller could hand to a split tile kernel
 // (0: none, no split).
-inline Choice choose(bool column_wise, int m, int n, int k, size_t workspace_capacity) {
+inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity) {
   Choice c{};
+  // One row, fp16, blocks along K, at most one workgroup per compute unit and a long K: the GEMV without MFMA
+  // (measured against the MFMA form on rotating weights, N = 4096: K = 8192 6.5 against 7.0 us, K = 11008
+  // 8.0 against 8.6, K = 14336 9.7 against 10.3; K = 4096 4.8 against 4.6 and every wider N: the MFMA form).
+  if (m == 1 && column_wise && !bf16 && n / 16 <= kComputeUnits && n >= 2048 && k >= 8192 &&
+      static_cast<size_t>(k) * 2 + 1024 <= kMaxLdsBytes) {
+    c.family = kFamilyValuGemv;
+    c.valu_rows = valu_gemv_rows(m);
+    c.valu_waves = valu_gemv_waves(k);
+    return c;
+  }
   if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k);
   c.t = tile_plan(column_wise, m, n, k, workspace_capacity);
   c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_estimate_us(c.t, k)) ? kFamilyStreaming : kFamilyTile;

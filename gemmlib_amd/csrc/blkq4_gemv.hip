@@ -162,6 +162,8 @@ hipError_t raise_lds_limit() {
 template <int BS, bool HAS_ZP, int R, int kWaves>
 int launch_dot(const blkq4_gemm_args* a) {
   const size_t lds = static_cast<size_t>(R) * a->k * 2 + static_cast<size_t>(kWaves) * R * 16 * 4;
+  if (a->launched_id != nullptr) *a->launched_id = valu_gemv_id(R, kWaves);
+  if (a->dry_run) return 0;
   if (lds > kMaxLdsBytes) return static_cast<int>(hipErrorInvalidValue);
   constexpr auto kernel = gemv_dot_kernel<BS, HAS_ZP, R, kWaves>;
   if (hipError_t e = raise_lds_limit<kernel>(); e != hipSuccess) return static_cast<int>(e);
@@ -174,18 +176,20 @@ int launch_dot(const blkq4_gemm_args* a) {
 
 template <int BS, bool HAS_ZP, int R>
 int launch_waves(const blkq4_gemm_args* a) {
-  // sixteen waves when every one of them gets at least two slices, else eight, else four
-  const int slices = (a->k / 32 + 3) / 4;
-  if (slices >= 32) return launch_dot<BS, HAS_ZP, R, 16>(a);
-  if (slices >= 16) return launch_dot<BS, HAS_ZP, R, 8>(a);
-  return launch_dot<BS, HAS_ZP, R, 4>(a);
+  switch (valu_gemv_waves(a->k)) {
+    case 16: return launch_dot<BS, HAS_ZP, R, 16>(a);
+    case 8: return launch_dot<BS, HAS_ZP, R, 8>(a);
+    default: return launch_dot<BS, HAS_ZP, R, 4>(a);
+  }
 }
 
 template <int BS, bool HAS_ZP>
 int launch_rows(const blkq4_gemm_args* a) {
-  if (a->m == 1) return launch_waves<BS, HAS_ZP, 1>(a);
-  if (a->m == 2) return launch_waves<BS, HAS_ZP, 2>(a);
-  return launch_waves<BS, HAS_ZP, 4>(a);
+  switch (valu_gemv_rows(a->m)) {
+    case 1: return launch_waves<BS, HAS_ZP, 1>(a);
+    case 2: return launch_waves<BS, HAS_ZP, 2>(a);
+    default: return launch_waves<BS, HAS_ZP, 4>(a);
+  }
 }
 
 template <int BS>
