@@ -83,27 +83,53 @@ DESCRIPTION = {
 # reads for the runtime's device-to-device copy of a 128 MiB buffer in the same run (FETCH_SIZE reads
 # 65 552 KiB for 131 072 KiB fetched: factor 2.0; WRITE_SIZE reads 131 072 KiB: factor 1.0).  The counters
 # sit between L2 and the memory fabric, so reads served by the Infinity Cache are included.  A script cannot
-# read these counters for itself; the figures are refreshed when a kernel changes.
+# read these counters for itself; the figures are refreshed when a kernel changes, and `traffic_kernel` in the
+# figure of a workload is reported only while the library still picks the kernel it was taken from (TRAFFIC_KERNEL).
 COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65552.0, "WRITE_SIZE": 1.0}
 COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
-    "C4": (44106.8, 16384.0),
-    "C2": (4416.0, 8.0),
-    "C3": (13870.4, 344.0),
-    "C5": (860484.2, 229376.0),
-    "C5_prepack": (229445.4, 158478.8),
-    "C4r": (44108.3, 16384.0),
-    "C2r": (4417.4, 8.0),
-    "C1": (865.1, 128.0),
-    "M128": (8653.7, 1024.0),
-    "V128K": (136437.3, 250.7),
-    "B16": (63847.2, 896.0),
-    "C4b": (44121.8, 16384.0),
-    "C2b": (4418.8, 8.0),
+    "C4": (44108.2, 16387.9),
+    "C2": (4428.6, 8.0),
+    "C3": (13882.7, 344.0),
+    "C5": (860369.0, 229403.7),
+    "C5_prepack": (229443.7, 157730.2),
+    "C4r": (44108.5, 16396.1),
+    "C2r": (4430.1, 8.0),
+    "C1": (866.0, 128.0),
+    "M128": (8649.1, 1024.0),
+    "M256": (24123.1, 11274.1),
+    "M512": (37925.6, 4545.3),
+    "M768N11K": (60847.5, 16513.6),
+    "M256K11K": (43356.1, 19403.8),
+    "V128K": (136363.9, 250.5),
+    "B16": (63817.2, 896.0),
+    "C4b": (44128.6, 16392.7),
+    "C2b": (4427.1, 8.0),
 }
 
 
-def traffic_bytes(name):
-    if name not in COUNTER_KIB:
+TRAFFIC_KERNEL = {  # what blkq4_gemm_plan_sm80 said the workload runs when its counters were taken
+    "C1": "streaming: 8 waves splitting K, 1 column tile(s) x 32 rows, 2 slices in flight, rows whole in LDS, 2 row group(s), 128 workgroups",
+    "C2": "streaming: 16 waves splitting K, 1 column tile(s) x 16 rows, 2 slices in flight, rows whole in LDS, 1 row group(s), 256 workgroups",
+    "C3": "streaming: 16 waves splitting K, 3 column tile(s) x 16 rows, 2 slices in flight, rows whole in LDS, 1 row group(s), 256 workgroups",
+    "C4": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
+    "C5": "tile: 256 x 256, 4 + 0 waves, 1792 tiles",
+    "C4r": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
+    "C2r": "streaming: 16 waves splitting K, 1 column tile(s) x 16 rows, 2 slices in flight, rows whole in LDS, 1 row group(s), 256 workgroups",
+    "M128": "streaming: 8 waves splitting K, 4 column tile(s) x 32 rows, 2 slices in flight, rows staged per slice, 4 row group(s), 256 workgroups",
+    "V128K": "streaming: 4 waves with column tiles of their own, 1 column tile(s) x 16 rows, 4 slices in flight, rows whole in LDS, 1 row group(s), 2016 workgroups (walking)",
+    "B16": "streaming: 4 waves splitting K, 4 column tile(s) x 16 rows, 2 slices in flight, rows staged per slice, 1 row group(s), 448 workgroups",
+    "C4b": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
+    "C2b": "streaming: 16 waves splitting K, 1 column tile(s) x 16 rows, 2 slices in flight, rows whole in LDS, 1 row group(s), 256 workgroups",
+    "M256": "tile: 64 x 128, 4 + 4 waves, 128 tiles, the last 128 in 2 parts (workspace 8404992 bytes)",
+    "M512": "tile: 64 x 128, 4 + 4 waves, 256 tiles",
+    "M768N11K": "tile: 256 x 256, 4 + 0 waves, 129 tiles",
+    "M256K11K": "tile: 128 x 128, 4 + 4 waves, 64 tiles, the last 64 in 4 parts (workspace 16793600 bytes)",
+}
+
+
+def traffic_bytes(name, kernel=None):
+    """HBM-side bytes per launch, or None when there is no figure or it was taken from another kernel."""
+    if name not in COUNTER_KIB or (name in TRAFFIC_KERNEL and kernel is not None and TRAFFIC_KERNEL[name] != kernel):
         return None
     f, w = COUNTER_KIB[name]
     return int(round((f * COUNTER_SCALE["FETCH_SIZE"] + w * COUNTER_SCALE["WRITE_SIZE"]) * 1024))
@@ -294,6 +320,7 @@ def bench_gemm(torch, capi, name, device, steps, warmup, with_cpu=True):
         return lambda: capi.gemm(bs, col, m, n, k, a, q_w, q_s, q_zp, out, bf16=name in BF16)
 
     launches = [mk(s) for s in sets]
+    kernel = capi.gemm_plan(bs, col, m, n, k, has_offsets, name in BF16)[2]
     # every weight set is visited equally often, and the last launch reads the last (seeded) set
     n_launch = copies * ((max(steps, copies) + copies - 1) // copies)
     wall, evt, mode = timed_region(torch, launches, n_launch, warmup)
@@ -308,12 +335,12 @@ def bench_gemm(torch, capi, name, device, steps, warmup, with_cpu=True):
     res = {
         "workload": DESCRIPTION[name], "value": round(value, 3), "unit": unit,
         "ms_per_step": round(per_call_wall * 1e3, 6), "kernel_us": round(per_call_evt * 1e6, 3),
-        "kernel": capi.gemm_plan(bs, col, m, n, k, has_offsets, name in BF16)[2],
+        "kernel": kernel,
         "timing": mode, "launches_per_region": n_launch, "weight_sets": copies,
         "weight_footprint_bytes": copies * per_set, "flops": flops, "bytes": nbytes,
         "tflops": round(flops / per_call_evt / 1e12, 3), "gbps": round(nbytes / per_call_evt / 1e9, 3),
         "roofline": {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": traffic_bytes(name)},
+                     "frac": round(achieved / peak, 4), "traffic": traffic_bytes(name, kernel)},
     }
     torch.cuda.synchronize()
     parity, base, _ = check_and_baseline(name, a, sets[-1], out, w_host, with_cpu)
@@ -503,9 +530,15 @@ def main(argv=None) -> int:
     ap.add_argument("--configs", default="C4,C2,C1,C3,C5,prepack,C4r,C2r,M128,M256,M512,M768N11K,M256K11K,V128K,B16,C4b,C2b")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-context", action="store_true", help="skip the floors and the library comparison")
+    ap.add_argument("--settle", type=float, default=None,
+                    help="seconds of untimed replay before the timed regions (default 0.4; profiling runs use less)")
     ap.add_argument("--gemv-forms", action="store_true",
                     help="only the A/B of the two forms of the GEMV (MFMA / no MFMA) over a list of shapes")
     args = ap.parse_args(argv)
+    if args.settle is not None:
+        global SETTLE_SECONDS
+        SETTLE_SECONDS = args.settle
+        timed_region.__defaults__ = (SETTLE_SECONDS, TIMED_REGIONS)
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
         return 2
