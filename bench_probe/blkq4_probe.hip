@@ -88,6 +88,13 @@ PROBE_EXPORT int blkq4_probe_empty(void* scratch, void* stream) {
   return static_cast<int>(hipGetLastError());
 }
 
+// an empty kernel of any launch shape (what a graph node costs depends on how many waves have to be started)
+PROBE_EXPORT int blkq4_probe_empty_shape(int grid, int block, int lds_bytes, void* scratch, void* stream) {
+  hipLaunchKernelGGL(empty_kernel, dim3(grid), dim3(block), lds_bytes, static_cast<hipStream_t>(stream),
+                     static_cast<unsigned*>(scratch));
+  return static_cast<int>(hipGetLastError());
+}
+
 // packed_w: uint8[K/32][N][16]; scales: fp16 [K/64][N] or NULL; scratch: at least N / 16 * 4 bytes
 PROBE_EXPORT int blkq4_probe_stream(const void* packed_w, const void* scales, int n, int k, void* scratch,
                                     void* stream) {
@@ -99,6 +106,23 @@ PROBE_EXPORT int blkq4_probe_stream(const void* packed_w, const void* scales, in
                        static_cast<unsigned*>(scratch), n, k);
   } else {
     hipLaunchKernelGGL((stream_kernel<8, false>), grid, block, 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint4*>(packed_w), static_cast<const uint16_t*>(nullptr),
+                       static_cast<unsigned*>(scratch), n, k);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+// the same requests from workgroups of sixteen waves (the product's shape for C2)
+PROBE_EXPORT int blkq4_probe_stream16(const void* packed_w, const void* scales, int n, int k, void* scratch,
+                                      void* stream) {
+  if (n % 16 != 0 || k % 64 != 0) return static_cast<int>(hipErrorInvalidValue);
+  const dim3 grid(n / 16), block(64 * 16);
+  if (scales) {
+    hipLaunchKernelGGL((stream_kernel<16, true>), grid, block, 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint4*>(packed_w), static_cast<const uint16_t*>(scales),
+                       static_cast<unsigned*>(scratch), n, k);
+  } else {
+    hipLaunchKernelGGL((stream_kernel<16, false>), grid, block, 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint4*>(packed_w), static_cast<const uint16_t*>(nullptr),
                        static_cast<unsigned*>(scratch), n, k);
   }
