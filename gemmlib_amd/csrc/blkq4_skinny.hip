@@ -203,56 +203,67 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
   Slot<BS, NT, MT, AM, ROW> slot[DEPTH];
 
-  // Rows to LDS, in the layout [unit][row][64 B]; requested before anything else.
-  uint32_t a_rd = 0;  // LDS byte offset of this lane's row inside a unit, chunk 0
-  uint32_t a_swz = 0;
+  // Rows to LDS, requested before anything else.  Layout: [pair of 32-deep units][row][128 B], the eight 16-byte
+  // chunks of a row's 128 bytes XOR-swizzled with bits 1..3 of the row (the 16 lanes of a fragment read touch 16
+  // rows at the same logical chunk and land on 16 different 16-byte slots of the 256 bytes the banks span).  A copy
+  // instruction moves 1 KiB = eight rows' 128 contiguous bytes each: whole 128-byte lines of the activations
+  // (with 64 bytes per row and instruction the staging of 16 rows cost 1 us more on C3's shape).  The LDS side of
+  // a copy is lane-linear, so the swizzle is applied to the global address a lane fetches.  A 128-deep slice is
+  // two pairs = 256 * rows contiguous bytes.
+  uint32_t a_rd = 0;   // LDS byte offset of this lane's row inside a pair
+  uint32_t a_swz = 0;  // bits 1..3 of the row
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
                             (__attribute__((address_space(3))) uint8_t*)(smem)));
   if (AM == kRowsPerSlotInLds) {
-    // this wave's slots: DEPTH pieces of [4 units][kSlotRows rows][64 B]
-    a_rd = (wave * DEPTH) * kSlotBytes + g * (kSlotRows * 64) + nl * 64;
-    a_swz = (nl >> 2) & 3;
+    // this wave's slots: DEPTH pieces of [2 pairs][kSlotRows rows][128 B]
+    a_rd = (wave * DEPTH) * kSlotBytes + nl * 128;
+    a_swz = (nl >> 1) & 7;
   }
   if (A_LDS) {
     const int rows = 1 << rows_log2;
     if (kSplit == 1) {
-      // every wave needs all of K: the waves share out the copies (copy q fills LDS bytes [1024 q, 1024 q + 1024)
-      // of the [unit][row][64 B] layout, lane l the 16 bytes at 16 l) and meet at a barrier below
+      // every wave needs all of K: the waves share out the copies (copy q fills LDS bytes [1024 q, 1024 q + 1024),
+      // lane l the 16 bytes at 16 l) and meet at a barrier below
       const int copies = ((K << rows_log2) + 511) >> 9;  // K * 2 * rows bytes in 1 KiB copies, the last one may be partial
       for (int q = wave; q < copies; q += kWaves) {
         const uint32_t off = q * 1024 + lane * 16;
-        const int u = min(static_cast<int>(off >> (6 + rows_log2)), units - 1);  // past the end: any valid unit
-        const int row = (off >> 6) & (rows - 1);
-        const int chunk = (lane & 3) ^ ((row >> 2) & 3);
-        async_copy_16(lds0 + q * 1024, A, (static_cast<uint32_t>(min(row, M - 1)) * K + u * 32 + chunk * 8) * 2);
+        const int e = off >> 7;
+        const int row = e & (rows - 1);
+        const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+        const int u = min(2 * (e >> rows_log2) + (chunk >> 2), units - 1);  // past the end: any valid unit
+        async_copy_16(lds0 + q * 1024, A, (static_cast<uint32_t>(min(row, M - 1)) * K + u * 32 + (chunk & 3) * 8) * 2);
       }
     } else {
       // The waves split K: a wave stages the rows of ITS slices, nobody else reads them, and no barrier is needed:
       // the copies are requested before the wave's first weights, requests complete in order, so a wave that has
-      // its first weights has all its rows (consume() makes its first reads wait for a weight word).  A slice
-      // is [4 units][rows][64 B] = 256 * rows contiguous bytes; with fewer than four rows a copy moves less than
-      // its 1 KiB (the lanes past the slice, or past the end of K in the last slice, are switched off).
+      // its first weights has all its rows (consume() makes its first reads wait for a weight word).  With fewer
+      // than four rows a copy moves less than its 1 KiB (the lanes past the slice, or past the end of K in the
+      // last slice, are switched off: K is a multiple of 64, so a pair exists whole or not at all).
       const uint32_t slice_bytes = 256u << rows_log2;
       for (int li = 0; li < my_slices; ++li) {
         const int sl = ws + kSplit * li;
         for (uint32_t off0 = 0; off0 < slice_bytes; off0 += 1024) {
           const uint32_t off = off0 + lane * 16;
-          const int u = 4 * sl + static_cast<int>(off >> (6 + rows_log2));
+          const int e = off >> 7;
+          const int row = e & (rows - 1);
+          const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+          const int u = 4 * sl + 2 * (e >> rows_log2) + (chunk >> 2);
           if (off < slice_bytes && u < units) {  // (units past the end of K are not read, and lie outside the rows' LDS)
-            const int row = (off >> 6) & (rows - 1);
-            const int chunk = (lane & 3) ^ ((row >> 2) & 3);
             async_copy_16(__builtin_amdgcn_readfirstlane(lds0 + (static_cast<uint32_t>(sl) << (8 + rows_log2)) + off0), A,
-                          (static_cast<uint32_t>(min(row, M - 1)) * K + u * 32 + chunk * 8) * 2);
+                          (static_cast<uint32_t>(min(row, M - 1)) * K + u * 32 + (chunk & 3) * 8) * 2);
           }
         }
       }
     }
-    const int row = min(nl, rows - 1);  // row tile mt: 16 mt rows further (same swizzle: bits 2..3 of the row)
-    a_rd = row * 64;
-    a_swz = (row >> 2) & 3;
+    const int row = min(nl, rows - 1);  // row tile mt: 16 mt rows further (same swizzle: bits 1..3 of the row)
+    a_rd = row * 128;
+    a_swz = (row >> 1) & 7;
   }
-  a_lane[0] = (static_cast<uint32_t>(g) << (6 + rows_log2)) + a_rd;
-  a_lane[1] = (static_cast<uint32_t>(g_alt) << (6 + rows_log2)) + a_rd;
+  // unit g of a slice is half g & 1 of pair g >> 1 (a_lane: offset of the pair's row; a_half: which 64 bytes)
+  const uint32_t pair_bytes = (AM == kRowsPerSlotInLds) ? kSlotRows * 128 : (128u << rows_log2);
+  a_lane[0] = static_cast<uint32_t>(g >> 1) * pair_bytes + a_rd;
+  a_lane[1] = static_cast<uint32_t>(g_alt >> 1) * pair_bytes + a_rd;
+  const uint32_t a_half[2] = {static_cast<uint32_t>(g & 1) * 4, static_cast<uint32_t>(g_alt & 1) * 4};
   // a slot past the end asks for valid units (so every slot always issues the same loads); its scales are
   // zeroed when the slot is consumed (not here: that would wait for the load right after requesting it),
   // which makes it contribute exactly 0
@@ -267,13 +278,13 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       /* copy q: LDS bytes [1024 q, 1024 q + 1024) of the slot, lane l the 16 bytes at 16 l; */ \
       /* requested before the slot's weights, so whoever has the weights has the rows        */ \
       _Pragma("unroll") for (int q = 0; q < 4 * MT; ++q) {                                     \
-        const int rr_ = 16 * q + (lane >> 2);            /* (unit, row) index inside the slot */ \
-        const int u_ = 4 * sl_ + rr_ / kSlotRows;                                              \
-        const int ug_ = (u_ < units) ? u_ : (u_ & wrap_mask);                                  \
+        const int rr_ = 8 * q + (lane >> 3);             /* (pair, row) index inside the slot */ \
         const int row_ = rr_ % kSlotRows;                                                      \
-        const int chunk_ = (lane & 3) ^ ((row_ >> 2) & 3);                                     \
+        const int chunk_ = (lane & 7) ^ ((row_ >> 1) & 7);                                     \
+        const int u_ = 4 * sl_ + 2 * (rr_ / kSlotRows) + (chunk_ >> 2);                        \
+        const int ug_ = (u_ < units) ? u_ : (u_ & wrap_mask);                                  \
         async_copy_16(__builtin_amdgcn_readfirstlane(lds0 + (wave * DEPTH + (d_)) * kSlotBytes + q * 1024), A, \
-                      (static_cast<uint32_t>(min(row_, M - 1)) * K + ug_ * 32 + chunk_ * 8) * 2); \
+                      (static_cast<uint32_t>(min(row_, M - 1)) * K + ug_ * 32 + (chunk_ & 3) * 8) * 2); \
       }                                                                                        \
     }                                                                                          \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                           \
@@ -419,19 +430,22 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
         const int sl_a = (kSplit == 1 || slice <= last_slice) ? sl : ws;
         const bool alt_a = rem != 0 && sl_a == last_slice;
         const uint8_t* ap = a_lds + (static_cast<uint32_t>(4 * sl_a) << (6 + rows_log2)) + (alt_a ? a_lane[1] : a_lane[0]) + arrived;
+        const uint32_t half = alt_a ? a_half[1] : a_half[0];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            af[mt][j] = *reinterpret_cast<const uint4*>(ap + mt * 1024 + ((j ^ a_swz) * 16));
+            af[mt][j] = *reinterpret_cast<const uint4*>(ap + mt * 2048 + (((half + j) ^ a_swz) * 16));
           }
       } else {
-        const uint8_t* ap = a_lds + a_rd + d * kSlotBytes + arrived;
+        // (all four units of a slot hold valid rows, also past the end of K: the lane reads its own unit g)
+        const uint8_t* ap = a_lds + a_lane[0] + d * kSlotBytes + arrived;
+        const uint32_t half = a_half[0];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            af[mt][j] = *reinterpret_cast<const uint4*>(ap + mt * 1024 + ((j ^ a_swz) * 16));
+            af[mt][j] = *reinterpret_cast<const uint4*>(ap + mt * 2048 + (((half + j) ^ a_swz) * 16));
           }
       }
 #pragma unroll
