@@ -29,7 +29,13 @@ LIB_PATH = os.path.join(LIB_DIR, "libms_blkq4gemm.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 HIP_SOURCES = ["blkq4_prepack.hip", "blkq4_skinny.hip", "blkq4_skinny_bf16.hip", "blkq4_gemm.hip", "blkq4_gemm_bf16.hip",
-               "blkq4_workspace.hip", "blkq4_gemv.hip"]
+               "blkq4_workspace.hip", "blkq4_gemv.hip", "blkq4_decode.hip", "blkq4_decode_bf16.hip"]
+# Kernel arguments of the decode kernels arrive in registers with the wave (the code object keeps a prologue that
+# loads them for firmware that does not preload).
+EXTRA_HIP_FLAGS = {
+    "blkq4_decode.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    "blkq4_decode_bf16.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+}
 HOST_SOURCES = ["blkq4_api.cpp"]
 
 # -ffp-contract=off: every fused multiply-add the quantizer needs is written as an explicit fmaf.
@@ -64,7 +70,7 @@ def build_library(verbose: bool = True) -> str:
     for src in HIP_SOURCES:
         obj = os.path.join(OBJ_DIR, src + ".o")
         objs.append(obj)
-        jobs.append(([HIPCC, *HIP_FLAGS, "-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj],
+        jobs.append(([HIPCC, *HIP_FLAGS, *EXTRA_HIP_FLAGS.get(src, []), "-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj],
                      "packed-fp32-ops"))
     for src in HOST_SOURCES:
         obj = os.path.join(OBJ_DIR, src + ".o")

@@ -181,7 +181,7 @@ extern "C" BLKQ4_EXPORT int blkq4_bf16_quant_sm80(int block_size, bool column_wi
 namespace {
 
 int launch_choice(const blkq4::Choice& choice, bool bf16, const blkq4_gemm_args* args) {
-  if (choice.family == blkq4::kFamilyValuGemv) return blkq4_dev_gemv_dot(args);
+  if (choice.family == blkq4::kFamilyDecode) return bf16 ? blkq4_dev_decode_bf16(args) : blkq4_dev_decode(args);
   const bool streaming = choice.family == blkq4::kFamilyStreaming;
   return bf16 ? (streaming ? blkq4_dev_skinny_bf16(args) : blkq4_dev_gemm_bf16(args))
               : (streaming ? blkq4_dev_skinny(args) : blkq4_dev_gemm(args));
@@ -326,6 +326,7 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
   }
   args.streaming = choice.s;
   args.tile = choice.t;
+  args.decode = choice.d;
   if (int code = launch_choice(choice, bf16, &args)) return device_failure(code, err);
   return 0;
 }
@@ -435,6 +436,7 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
   args.c = dummy;
   args.streaming = choice.s;
   args.tile = choice.t;
+  args.decode = choice.d;
   args.dry_run = 1;
   uint64_t launched = 0;
   args.launched_id = &launched;
@@ -444,9 +446,11 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
   if (launched_id != nullptr) *launched_id = launched;
   if (description != nullptr && description_size > 0) {
     std::string text;
-    if (choice.family == blkq4::kFamilyValuGemv) {
-      text = "gemv without MFMA: " + std::to_string(choice.valu_waves) + " waves splitting K, 16 columns x " +
-             std::to_string(choice.valu_rows) + " row(s), " + std::to_string(n / 16) + " workgroups";
+    if (choice.family == blkq4::kFamilyDecode) {
+      const auto& d = choice.d;
+      text = "decode: " + std::to_string(d.waves) + " waves splitting K, " + std::to_string(d.depth) +
+             " slices requested by each, " + std::to_string(d.nt) + " column tile(s) x " + std::to_string(d.rows) +
+             " row(s), " + std::to_string(d.grid) + " workgroups";
     } else if (streaming) {
       const auto& p = choice.s;
       text = "streaming: " + std::to_string(p.waves) + " waves" + (p.split == 1 ? " with column tiles of their own" : " splitting K") +

@@ -26,16 +26,17 @@ constexpr int kRowsPerSlotInLds = 2;  // 16 * MT rows x 128 k staged per slot, p
 
 constexpr int kFamilyStreaming = 0;  // weight-streaming kernel (blkq4_skinny.hip)
 constexpr int kFamilyTile = 1;       // MFMA tile kernel (blkq4_gemm.hip)
-constexpr int kFamilyValuGemv = 2;   // GEMV without MFMA (blkq4_gemv.hip)
+constexpr int kFamilyDecode = 2;     // decode kernel (blkq4_decode.hip)
 
 using StreamingShape = blkq4_streaming_plan;  // see blkq4_device.h
 using TileShape = blkq4_tile_plan;
+using DecodeShape = blkq4_decode_plan;
 
 struct Choice {
   int family;
   StreamingShape s;
   TileShape t;
-  int valu_rows, valu_waves;  // kFamilyValuGemv
+  DecodeShape d;
 };
 
 // A kernel's identity as one number: what choose() picked and what a launcher started can be compared.
@@ -49,7 +50,8 @@ inline uint64_t tile_id(int rt, int nt, int wm, int wn, int pw, bool split) {
          static_cast<uint64_t>(wm) << 24 | static_cast<uint64_t>(wn) << 16 | static_cast<uint64_t>(pw) << 8 |
          (split ? 1u : 0u);
 }
-// the GEMV without MFMA: rows kept (1, 2 or 4) and waves of a workgroup
+// the GEMV without MFMA (blkq4_gemv.hip; run only when asked for by name): rows kept (1, 2 or 4) and waves of a
+// workgroup
 inline int valu_gemv_rows(int m) { return m == 1 ? 1 : m == 2 ? 2 : 4; }
 inline int valu_gemv_waves(int k) {
   // sixteen waves when every one of them gets at least two 128-deep slices, else eight, else four
@@ -59,11 +61,55 @@ inline int valu_gemv_waves(int k) {
 inline uint64_t valu_gemv_id(int rows, int waves) {
   return 3ull << 60 | static_cast<uint64_t>(rows) << 8 | static_cast<uint64_t>(waves);
 }
+inline uint64_t decode_id(int rows, int nt, int waves, int depth) {
+  return 4ull << 60 | static_cast<uint64_t>(rows) << 24 | static_cast<uint64_t>(nt) << 16 |
+         static_cast<uint64_t>(waves) << 8 | static_cast<uint64_t>(depth);
+}
 inline uint64_t choice_id(const Choice& c) {
-  if (c.family == kFamilyValuGemv) return valu_gemv_id(c.valu_rows, c.valu_waves);
+  if (c.family == kFamilyDecode) return decode_id(c.d.rows, c.d.nt, c.d.waves, c.d.depth);
   return c.family == kFamilyStreaming
              ? streaming_id(c.s.depth, c.s.nt, c.s.mt, c.s.waves, c.s.am, c.s.split, c.s.refill != 0)
              : tile_id(c.t.rt, c.t.nt, c.t.wm, c.t.wn, c.t.pw, c.t.split_k > 1);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Decode kernel
+// ---------------------------------------------------------------------------------------------------------
+
+constexpr int kDecodeMaxRows = 4;
+constexpr int kDecodeMaxDepth = 8;
+
+// LDS of a workgroup: the rows of every wave's slices (256 bytes per row and slice), then the waves' partial
+// tiles (64 bytes per row and tile)
+inline size_t decode_lds_bytes(int rows, int nt, int waves, int depth) {
+  return static_cast<size_t>(waves) * depth * 256 * rows + static_cast<size_t>(waves) * nt * rows * 64;
+}
+
+// The decode kernel's shape for m rows, or false when it has none: blocks along K, at most kDecodeMaxRows rows,
+// K in whole 128-deep slices, few enough of them for 16 waves to request them all at once, and packed weights that
+// 32-bit offsets reach.  Eight waves by default (measured on M = 1, rotating weights, against 4 and 16 waves:
+// K = 2048, N = 2048: 2.62 against 2.74 and 2.68 us; K = 4096, N = 11008: 6.54 against 6.64 and 7.06;
+// N = 128256: 49.1 against 50.2 and 58.3; K = 8192, N = 4096: 5.41 against 16 waves' 5.40), four for short K, and
+// for one workgroup per compute unit at most when they then request eight slices each (K = 4096, N = 4096: 3.68
+// against 3.82 and 3.84 us), sixteen when eight would have to request more than eight slices each.
+inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) {
+  if (!column_wise || m < 1 || m > kDecodeMaxRows || (k % 128) != 0 || (n % 16) != 0 ||
+      static_cast<uint64_t>(k) * static_cast<uint64_t>(n) > (uint64_t{1} << 32)) {
+    return false;
+  }
+  const int slices = k / 128;
+  const int tiles = n / 16;
+  int waves = 8;
+  if (slices <= 8 || (slices > 24 && slices <= 32 && tiles <= kComputeUnits)) waves = 4;
+  if (slices > 8 * kDecodeMaxDepth) waves = 16;
+  if (slices > 16 * kDecodeMaxDepth) return false;
+  d->rows = m == 1 ? 1 : 4;
+  d->nt = 1;
+  d->waves = waves;
+  d->depth = (slices + waves - 1) / waves;
+  d->grid = static_cast<uint32_t>((tiles + d->nt - 1) / d->nt);
+  d->lds_bytes = static_cast<uint32_t>(decode_lds_bytes(d->rows, d->nt, d->waves, d->depth));
+  return d->lds_bytes <= kMaxLdsBytes;
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -396,15 +442,11 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
 // The whole decision.  workspace_capacity: bytes of workspace the caller could hand to a split tile kernel
 // (0: none, no split).
 inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity) {
+  (void)bf16;  // the same shapes for both element types
   Choice c{};
-  // One row, fp16, blocks along K, at most one workgroup per compute unit and a long K: the GEMV without MFMA
-  // (measured against the MFMA form on rotating weights, N = 4096: K = 8192 6.5 against 7.0 us, K = 11008
-  // 8.0 against 8.6, K = 14336 9.7 against 10.3; K = 4096 4.8 against 4.6 and every wider N: the MFMA form).
-  if (m == 1 && column_wise && !bf16 && n / 16 <= kComputeUnits && n >= 2048 && k >= 8192 &&
-      static_cast<size_t>(k) * 2 + 1024 <= kMaxLdsBytes) {
-    c.family = kFamilyValuGemv;
-    c.valu_rows = valu_gemv_rows(m);
-    c.valu_waves = valu_gemv_waves(k);
+  // few rows, blocks along K, a K that a workgroup can request at once: the decode kernel
+  if (decode_shape(column_wise, m, n, k, &c.d)) {
+    c.family = kFamilyDecode;
     return c;
   }
   if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k);

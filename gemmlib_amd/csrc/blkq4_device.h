@@ -70,6 +70,15 @@ typedef struct {
   size_t workspace_bytes; /* arrival counters + partial tiles, 0 without a split */
 } blkq4_tile_plan;
 
+/* Which decode kernel runs (blkq4_decode.hip): `rows` activation rows kept (a power of two >= m), `nt` column
+ * tiles per workgroup, `waves` waves that split K, `depth` slices requested by each.  Filled in by
+ * blkq4::decode_shape() (blkq4_choose.h). */
+typedef struct {
+  int rows, nt, waves, depth;
+  uint32_t grid;       /* workgroups */
+  uint32_t lds_bytes;  /* dynamic LDS */
+} blkq4_decode_plan;
+
 typedef struct {
   int block_size;
   int column_wise;          /* as in blkq4_prepack_args */
@@ -83,6 +92,7 @@ typedef struct {
   void* stream;
   blkq4_streaming_plan streaming; /* read by blkq4_dev_skinny* */
   blkq4_tile_plan tile;           /* read by blkq4_dev_gemm* */
+  blkq4_decode_plan decode;       /* read by blkq4_dev_decode* */
   void* workspace;                /* tile.split_k > 1: device memory of workspace_bytes, 256-byte aligned, whose */
   size_t workspace_bytes;         /* first 16 KiB (the arrival counters) are zero between launches */
   int dry_run;                    /* 1: launch nothing, only report the kernel */
@@ -102,6 +112,8 @@ int blkq4_dev_gemm(const blkq4_gemm_args* args);   /* MFMA tile kernel, every m 
 int blkq4_dev_skinny(const blkq4_gemm_args* args); /* weight-streaming kernel, 1 <= m <= 1024 */
 int blkq4_dev_gemm_bf16(const blkq4_gemm_args* args);   /* the tile kernel with bf16 a, scales, c and bias */
 int blkq4_dev_skinny_bf16(const blkq4_gemm_args* args); /* the same with bf16 a, scales, c and bias */
+int blkq4_dev_decode(const blkq4_gemm_args* args);      /* decode kernel: few rows, all of K requested at once, blocks along K */
+int blkq4_dev_decode_bf16(const blkq4_gemm_args* args); /* the same with bf16 a, scales, c and bias */
 int blkq4_dev_gemv_dot(const blkq4_gemm_args* args);    /* fp16 GEMV on the vector ALU (no MFMA): 1 <= m <= 4, blocks along K */
 int blkq4_dev_repack(const blkq4_repack_args* args);
 const char* blkq4_dev_error_string(int code);

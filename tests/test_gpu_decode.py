@@ -1,0 +1,115 @@
+"""The decode kernel (gemmlib_amd/csrc/blkq4_decode.hip: 1 to 4 rows, blocks along K, all of K requested at once),
+through blkq4_fp16_gemm_sm80 / blkq4_bf16_gemm_sm80, against the oracle: the reference's exact construction bit
+for bit (test/blkq4_fp16_gemm_sm80_test.cu:194-256,469-472) for every block size, with and without zero-points,
+every number of slices per wave from 1 to 8, slice counts that do not divide among the waves (the last slot of
+some waves stays empty), every wave count, N that is a multiple of 32 and nothing more; Gaussian data within
+1e-2; the bias in the epilogue; the same bits on every call."""
+
+import numpy as np
+import pytest
+import torch
+
+from bf16_util import bf16_kat, grid_activations_bf16
+from gpu_util import max_rel_err, quantize_on_gpu, to_dev, to_np
+from test_gpu_bf16 import dev_to_bits, gaussian_bits, gemm_bf16, quantize_bf16
+from test_gpu_gemm import gaussian_problem, grid_activations
+
+pytestmark = pytest.mark.gpu
+
+# (bs, zero-points, m, n, k): k / 128 slices over 4, 8 or 16 waves
+EXACT_CASES = [
+    (64, False, 1, 4096, 4096),    # 4 waves x 8
+    (64, True, 1, 4128, 4096),     # 8 waves x 4, 258 workgroups
+    (32, True, 2, 1024, 128),      # one slice: three of four waves have none
+    (16, True, 3, 160, 256), (64, False, 4, 64, 384), (32, False, 1, 96, 640), (16, False, 2, 1056, 1024),
+    (64, True, 1, 2048, 1152),     # 9 slices over 8 waves: depth 2, seven waves with an empty slot
+    (32, True, 4, 544, 2048), (16, True, 1, 288, 2176), (64, False, 3, 320, 3072), (32, True, 1, 4096, 3200),
+    (64, True, 2, 1024, 5120), (16, False, 1, 512, 6144), (32, False, 4, 2080, 7168), (64, True, 1, 4096, 8192),
+    (64, False, 1, 1024, 8320),    # 65 slices: 16 waves x 5, one full
+    (32, True, 3, 704, 11008), (16, True, 1, 256, 12288), (64, False, 2, 128, 14336), (64, True, 4, 32, 16384),
+    (32, False, 1, 128256, 512),   # many workgroups
+]
+
+
+def _run(capi, device, bs, a, q_w, q_s, q_zp, n, **kw):
+    m, k = a.shape
+    out = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+    capi.gemm(bs, True, m, n, k, to_dev(a, device), q_w, q_s, q_zp, out, **kw)
+    torch.cuda.synchronize()
+    return to_np(out)
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", EXACT_CASES)
+def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
+    assert capi.gemm_plan(bs, True, m, n, k, has_offsets)[2].startswith("decode:")
+    rng = np.random.default_rng(m * 131 + n * 17 + k + bs + has_offsets)
+    kat = oracle.kat_generate(bs, True, k, n, has_offsets)
+    a = grid_activations(rng, m, k)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, kat["weights"], has_offsets)
+    ref = oracle.gemm(a, kat["weights"])
+    got = _run(capi, device, bs, a, q_w, q_s, q_zp, n)
+    if not np.array_equal(got.view(np.uint16), ref.view(np.uint16)):
+        bad = np.argwhere(got.view(np.uint16) != ref.view(np.uint16))
+        raise AssertionError(f"{bad.shape[0]} of {m * n} outputs differ, first {bad[:5].tolist()}")
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", [c for i, c in enumerate(EXACT_CASES) if i % 2 == 0 and c[3] <= 8192])
+def test_exact_on_known_answer_construction_in_bf16(oracle, capi, device, bs, has_offsets, m, n, k):
+    assert capi.gemm_plan(bs, True, m, n, k, has_offsets, bf16=True)[2].startswith("decode:")
+    rng = np.random.default_rng(m * 131 + n * 17 + k + bs + has_offsets)
+    kat = bf16_kat(oracle, bs, k, n, has_offsets, seed=m + n + k)
+    a = grid_activations_bf16(oracle, rng, m, k)
+    q_w, q_s, q_zp = quantize_bf16(capi, device, bs, kat["weights"], has_offsets)
+    got = gemm_bf16(capi, device, bs, a, q_w, q_s, q_zp, n)
+    ref = oracle.gemm(a, kat["weights"], bf16=True)
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", [
+    (64, False, 1, 4096, 4096), (32, True, 4, 11008, 4096), (16, True, 2, 2048, 8192), (64, True, 1, 4096, 11008),
+    (32, False, 3, 14336, 1152), (64, False, 1, 128256, 4096),
+])
+def test_gaussian_within_tolerance_same_bits_every_call(oracle, capi, device, bs, has_offsets, m, n, k):
+    a, w = gaussian_problem(5 + m + n + k, m, n, k)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, w, has_offsets)
+    canon, s, z = oracle.quantize(bs, True, w, has_offsets)
+    ref = oracle.gemm(a, oracle.dequantize(bs, True, canon, s, z))
+    got = _run(capi, device, bs, a, q_w, q_s, q_zp, n)
+    assert max_rel_err(got, ref) <= 1e-2
+    for _ in range(3):
+        again = _run(capi, device, bs, a, q_w, q_s, q_zp, n)
+        assert np.array_equal(again.view(np.uint16), got.view(np.uint16))
+    if m <= 4 and k * (4 if m > 2 else m) * 2 <= 150 * 1024:
+        other = _run(capi, device, bs, a, q_w, q_s, q_zp, n, valu=True)   # the GEMV without MFMA: same weights,
+        assert max_rel_err(got, other) <= 2e-3                           # fp32 sums in another order
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, True, 1, 4096, 4096), (16, True, 4, 2080, 1152)])
+def test_gaussian_in_bf16(oracle, capi, device, bs, has_offsets, m, n, k):
+    a, w = gaussian_bits(oracle, 77 + m + n + k, m, n, k)
+    q_w, q_s, q_zp = quantize_bf16(capi, device, bs, w, has_offsets)
+    canon, s, z = oracle.quantize(bs, True, w, has_offsets, bf16=True)
+    ref = oracle.gemm(a, oracle.dequantize(bs, True, canon, s, z, bf16=True), bf16=True)
+    got = gemm_bf16(capi, device, bs, a, q_w, q_s, q_zp, n)
+    assert max_rel_err(oracle.bf16_to_f32(got), oracle.bf16_to_f32(ref)) <= 1e-2
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, False, 1, 4096, 4096), (32, True, 3, 1056, 1152), (16, True, 4, 2048, 8192)])
+def test_bias_in_the_epilogue_equals_a_separate_add(oracle, capi, device, bs, has_offsets, m, n, k):
+    """as the reference module adds it (python/ms_blkq4linear.py:26-27): to the rounded output, in the tensor
+    library's way of adding two 16-bit tensors"""
+    a, w = gaussian_problem(m + n + k, m, n, k)
+    g = torch.Generator(device="cpu").manual_seed(n)
+    bias = (torch.randn(n, generator=g) * 0.5).to(torch.float16).to(device)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, w, has_offsets)
+    plain = torch.from_numpy(_run(capi, device, bs, a, q_w, q_s, q_zp, n).view(np.int16)).to(device).view(torch.float16)
+    fused = _run(capi, device, bs, a, q_w, q_s, q_zp, n, bias=bias)
+    plain += bias
+    assert np.array_equal(fused.view(np.uint16), to_np(plain).view(np.uint16))
+    ab, wb = gaussian_bits(oracle, m + n + k, m, n, k)
+    bias_b = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16).to(device)
+    q_w, q_s, q_zp = quantize_bf16(capi, device, bs, wb, has_offsets)
+    plain = torch.from_numpy(gemm_bf16(capi, device, bs, ab, q_w, q_s, q_zp, n).view(np.int16)).to(device).view(torch.bfloat16)
+    fused = gemm_bf16(capi, device, bs, ab, q_w, q_s, q_zp, n, bias=bias_b)
+    plain += bias_b
+    assert np.array_equal(fused, dev_to_bits(plain))
