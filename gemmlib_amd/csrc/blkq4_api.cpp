@@ -450,7 +450,7 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
       const auto& d = choice.d;
       text = "decode: " + std::to_string(d.waves) + " waves splitting K, " + std::to_string(d.depth) +
              " slices requested by each, " + std::to_string(d.nt) + " column tile(s) x " + std::to_string(d.rows) +
-             " row(s), " + std::to_string(d.grid) + " workgroups";
+             " row(s), " + std::to_string((n / 16 + d.nt - 1) / d.nt) + " workgroups";
     } else if (streaming) {
       const auto& p = choice.s;
       text = "streaming: " + std::to_string(p.waves) + " waves" + (p.split == 1 ? " with column tiles of their own" : " splitting K") +

@@ -76,7 +76,7 @@ inline uint64_t choice_id(const Choice& c) {
 // Decode kernel
 // ---------------------------------------------------------------------------------------------------------
 
-constexpr int kDecodeMaxRows = 4;
+constexpr int kDecodeMaxRows = 16;
 constexpr int kDecodeMaxDepth = 8;
 
 // LDS of a workgroup: the rows of every wave's slices (256 bytes per row and slice), then the waves' partial
@@ -85,13 +85,33 @@ inline size_t decode_lds_bytes(int rows, int nt, int waves, int depth) {
   return static_cast<size_t>(waves) * depth * 256 * rows + static_cast<size_t>(waves) * nt * rows * 64;
 }
 
-// The decode kernel's shape for m rows, or false when it has none: blocks along K, at most kDecodeMaxRows rows,
-// K in whole 128-deep slices, few enough of them for 16 waves to request them all at once, and packed weights that
-// 32-bit offsets reach.  Eight waves by default (measured on M = 1, rotating weights, against 4 and 16 waves:
-// K = 2048, N = 2048: 2.62 against 2.74 and 2.68 us; K = 4096, N = 11008: 6.54 against 6.64 and 7.06;
-// N = 128256: 49.1 against 50.2 and 58.3; K = 8192, N = 4096: 5.41 against 16 waves' 5.40), four for short K, and
-// for one workgroup per compute unit at most when they then request eight slices each (K = 4096, N = 4096: 3.68
-// against 3.82 and 3.84 us), sixteen when eight would have to request more than eight slices each.
+// Workgroups: one per group of nt column tiles, rounded up to whole sets of 64 groups (the kernel hands eight
+// neighbouring groups to each of the 8 XCDs in turn)
+inline uint32_t decode_grid(int n, int nt) {
+  const int groups = (n / 16 + nt - 1) / nt;
+  return static_cast<uint32_t>((groups + 63) / 64 * 64);
+}
+
+// The decode kernel's shape for m rows, or false when it has none or the streaming kernel is expected to be
+// faster: blocks along K, at most kDecodeMaxRows rows, K in whole 128-deep slices, few enough of them for the waves
+// to request them all at once and for the rows to fit in LDS, and packed weights that 32-bit offsets reach.
+//
+// Waves.  Eight by default (measured on M = 1, rotating weights, against 4 and 16 waves: K = 2048, N = 2048: 2.62
+// against 2.74 and 2.68 us; K = 4096, N = 11008: 6.54 against 6.64 and 7.06; N = 128256: 49.1 against 50.2 and 58.3;
+// K = 8192, N = 4096: 5.41 against 16 waves' 5.40), four for short K, and for one workgroup per compute unit at most
+// when they then request eight slices each (K = 4096, N = 4096: 3.68 against 3.74 and 3.80 us), sixteen when eight
+// would have to request more than eight slices each (up to four rows only).
+//
+// Column tiles per workgroup.  The busiest compute unit works through ceil(workgroups / 256) workgroups of nt
+// tiles each, and every workgroup costs a fraction of a tile's work on top: staging the rows, the instructions
+// before the first request, the sum across the waves.  That fraction, fitted to sweeps over N = 4096 .. 28672 at
+// K = 4096 and 8192: 0.1 for one row, 0.5 for more.  Two tiles with more than four slices per wave take a tenth
+// longer than that (registers: fewer workgroups fit a compute unit).
+//
+// Eight and sixteen rows keep 64 to 128 KiB of rows per workgroup, so one or two workgroups fit a compute unit and a
+// second round of them starts from nothing; once there are more rounds than that the streaming kernel, whose
+// workgroups keep their rows and walk over the column tiles, is faster (M = 16, K = 4096, N = 28672: 17.2 against
+// 20.9 us; M = 8, K = 8192, N = 14336: 15.5 against 18.4; but M = 16, K = 4096, N = 11008: 9.2 against 7.9).
 inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) {
   if (!column_wise || m < 1 || m > kDecodeMaxRows || (k % 128) != 0 || (n % 16) != 0 ||
       static_cast<uint64_t>(k) * static_cast<uint64_t>(n) > (uint64_t{1} << 32)) {
@@ -99,17 +119,42 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
   }
   const int slices = k / 128;
   const int tiles = n / 16;
+  const int rows = m == 1 ? 1 : m <= 4 ? 4 : m <= 8 ? 8 : 16;
   int waves = 8;
-  if (slices <= 8 || (slices > 24 && slices <= 32 && tiles <= kComputeUnits)) waves = 4;
-  if (slices > 8 * kDecodeMaxDepth) waves = 16;
-  if (slices > 16 * kDecodeMaxDepth) return false;
-  d->rows = m == 1 ? 1 : 4;
-  d->nt = 1;
+  if (rows <= 4) {
+    if (slices <= 8 || (slices > 24 && slices <= 32 && tiles <= kComputeUnits)) waves = 4;
+    if (slices > 8 * kDecodeMaxDepth) waves = 16;
+    if (slices > 16 * kDecodeMaxDepth) return false;
+  }
+  const int depth = (slices + waves - 1) / waves;
+  if (depth > ((rows == 16) ? 4 : kDecodeMaxDepth)) return false;
+  const int max_nt = rows >= 8 ? 3 : (waves == 8 ? 2 : 1);  // the instantiations that exist
+  const float per_workgroup = rows == 1 ? 0.1f : 0.5f;
+  int nt = 1;
+  float best = 0.f;
+  for (int t = 1; t <= max_nt; ++t) {
+    if (decode_lds_bytes(rows, t, waves, depth) > kMaxLdsBytes) break;
+    const int wgs = (tiles + t - 1) / t;
+    float cost = static_cast<float>((wgs + kComputeUnits - 1) / kComputeUnits) * (static_cast<float>(t) + per_workgroup);
+    if (rows <= 4 && t == 2 && depth > 4) cost *= 1.1f;
+    if (t == 1 || cost < best) {
+      best = cost;
+      nt = t;
+    }
+  }
+  d->rows = rows;
+  d->nt = nt;
   d->waves = waves;
-  d->depth = (slices + waves - 1) / waves;
-  d->grid = static_cast<uint32_t>((tiles + d->nt - 1) / d->nt);
-  d->lds_bytes = static_cast<uint32_t>(decode_lds_bytes(d->rows, d->nt, d->waves, d->depth));
-  return d->lds_bytes <= kMaxLdsBytes;
+  d->depth = depth;
+  d->grid = decode_grid(n, nt);
+  d->lds_bytes = static_cast<uint32_t>(decode_lds_bytes(rows, nt, waves, depth));
+  if (d->lds_bytes > kMaxLdsBytes) return false;
+  if (rows >= 8) {
+    const int per_unit = static_cast<size_t>(d->lds_bytes) * 2 <= kMaxLdsBytes ? 2 : 1;  // workgroups a compute unit holds
+    const int rounds = ((tiles + nt - 1) / nt + kComputeUnits * per_unit - 1) / (kComputeUnits * per_unit);
+    if (rounds > per_unit) return false;
+  }
+  return true;
 }
 
 // ---------------------------------------------------------------------------------------------------------

@@ -22,7 +22,9 @@
 //     (asynchronous global_load_lds copies, laid out [pair of 32-deep units][row][128 bytes], 16-byte chunks
 //     XOR-swizzled with bits 1..3 of the row: fragment reads without bank conflicts); its reads wait for the
 //     first weights and need no barrier;
-//   - one barrier: the waves' partial tiles meet in LDS and are summed in the order of the waves.
+//   - one barrier: the waves' partial tiles meet in LDS and are summed in the order of the waves;
+//   - neighbouring column tiles run on the same XCD at about the same time and share the cache lines of their
+//     scales and zero-points (16 columns use 32 and 16 bytes of a row).
 // Dequantization is the streaming kernel's (blkq4_dequant.h: one rounding per weight), accumulation fp32 in
 // v_mfma_f32_16x16x32_{f16,bf16} with the weights as the row operand.
 
@@ -99,19 +101,31 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
   const int slices = K >> 7;
   const int units = K >> 5;
   const int tiles = N >> 4;
+  // Workgroup -> group of NT column tiles.  Consecutive workgroups go to consecutive XCDs (8 of them, each with an L2
+  // of its own); an XCD's workgroups take eight neighbouring groups at a time, which share the cache lines of the
+  // zero-point and scale rows, so that those are fetched from memory once.  The grid is rounded up to whole sets
+  // of 64 groups.  (M = 1, K = N = 4096, one group per workgroup in launch order against two, four and eight
+  // neighbours per XCD: 3.66, 3.64, 3.78, 3.62 us; with zero-points 4.05, 3.71, 3.86, 3.69; blocks of 16 with
+  // zero-points 5.83, 4.80, 4.64, 4.52; no shape lost more than 2 %.)
+  const uint32_t wg = blockIdx.x;
+  const uint32_t cg = (((wg >> 3) >> 3) << 6) + ((wg & 7) << 3) + ((wg >> 3) & 7);
+  if (cg >= static_cast<uint32_t>((tiles + NT - 1) / NT)) return;
   // this wave's slices: s0 .. s0 + mine - 1, mine = D or D - 1
   const int s0 = (wave * slices) >> kLgWaves;
   const int mine = (((wave + 1) * slices) >> kLgWaves) - s0;
   const bool last_ok = mine == D;  // wave-uniform
 
-  // Rows first.  Copy q fills LDS bytes [1024 q, 1024 q + 1024) of the wave's part, lane l the 16 bytes at 16 l:
-  // row-chunk e = (pair, row), physical chunk l & 7 holds logical chunk (l & 7) ^ bits 1..3 of the row.  Units
-  // past the end of K (the missing slot of the last wave) fetch the last unit instead: any finite values do,
-  // they meet a zero scale.
+  // Rows.  A copy instruction fills 1 KiB of LDS, lane l the 16 bytes at 16 l: eight row-chunks e = (pair, row) of
+  // 128 bytes, physical chunk l & 7 holding logical chunk (l & 7) ^ bits 1..3 of the row.
+  // Up to four rows: all copies of the wave first (copy q fills bytes [1024 q, 1024 q + 1024) of the wave's part;
+  // a slice has less than a copy's worth of rows).  Units past the end of K (the missing slot of the last wave)
+  // fetch the last unit instead: any finite values do, they meet a zero scale.
+  // Eight or sixteen rows: a slot's copies (two or four) go right before the slot's other requests, see below.
+  constexpr bool kPerSlot = R >= 8;
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)(smem)));
   const uint32_t wave_lds = lds0 + wave * kWaveBytes;
 #pragma unroll
-  for (int q = 0; q < kCopies; ++q) {
+  for (int q = 0; q < (kPerSlot ? 0 : kCopies); ++q) {
     const uint32_t off = q * 1024 + lane * 16;
     const uint32_t e = off >> 7;
     const uint32_t r = e & (R - 1);
@@ -136,10 +150,24 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
     const uint32_t w_stride = static_cast<uint32_t>(N) * 64u;               // bytes: 4 units of N columns
     const uint32_t m_stride = static_cast<uint32_t>(N) * (128u / BS);       // elements: the blocks of a slice
     const uint32_t last = static_cast<uint32_t>(min(D - 1, slices - 1 - s0));  // the missing slot asks for the last slice again
+    // per-slot copies: copy h of a slot covers row-chunks 8 h .. 8 h + 7 of the slice; the lane's part of the
+    // address never changes, the slice adds 256 bytes along K
+    constexpr int kSlotCopies = kPerSlot ? R / 4 : 1;
+    uint32_t a_off[kSlotCopies];
+    if constexpr (kPerSlot) {
+#pragma unroll
+      for (int h = 0; h < kSlotCopies; ++h) {
+        const uint32_t e = 8 * h + (lane >> 3);
+        const uint32_t r = e & (R - 1);
+        const uint32_t chunk = (lane & 7) ^ ((r >> 1) & 7);
+        a_off[h] = (min(r, static_cast<uint32_t>(M - 1)) * K + (2 * (e >> kLgR) + (chunk >> 2)) * 32 + (chunk & 3) * 8) * 2 +
+                   static_cast<uint32_t>(s0) * 256u;
+      }
+    }
     uint32_t w_off[NT], m_idx[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      const uint32_t tile = (NT == 1) ? blockIdx.x : min(static_cast<uint32_t>(blockIdx.x * NT + t), static_cast<uint32_t>(tiles - 1));
+      const uint32_t tile = (NT == 1) ? cg : min(cg * NT + t, static_cast<uint32_t>(tiles - 1));
       const uint32_t col = tile * 16 + nl;
       w_off[t] = (unit0 * N + col) * 16u;
       m_idx[t] = blk0 * N + col;
@@ -147,6 +175,10 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       const uint32_t dd = (d == D - 1) ? last : static_cast<uint32_t>(d);
+      if constexpr (kPerSlot) {
+#pragma unroll
+        for (int h = 0; h < kSlotCopies; ++h) async_copy_16(wave_lds + d * kSliceBytes + h * 1024, A, a_off[h] + dd * 256u);
+      }
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -172,28 +204,38 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
   for (int t = 0; t < NT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   // This lane's fragment addresses: row nl (rows past R - 1 read row R - 1: their sums are not stored), unit g =
-  // half g & 1 of pair g >> 1.  The copies were requested before the first weights and requests complete in
-  // order: the reads wait for a word of the first weights, and with it for every row of this wave.
+  // half g & 1 of pair g >> 1.  The copies of a slot (of all slots, up to four rows) were requested before the
+  // slot's weights (the first slot's) and requests complete in order: the reads wait for a word of those weights,
+  // and with it for the rows.
   const uint32_t row = (R == 16) ? nl : min(nl, R - 1);
-  const uint32_t a_base = wave_lds + (g >> 1) * (128 * R) + row * 128 + zero_once_loaded(w[0][0].x);
   // logical chunk 4 (g & 1) + j lies at physical chunk c0 ^ j; with one or two rows nothing is swizzled
   const uint32_t c0 = ((g & 1) * 4) ^ ((row >> 1) & 7);
-  uint32_t a_rd[4];
+  const uint32_t a_lane = (wave_lds + (g >> 1) * (128 * R) + row * 128) | (c0 << 4);
+  auto fragments = [&](uint4 (&af)[4], int d, uint32_t arrived) {
+    const uint32_t base = a_lane + arrived;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) a_rd[j] = (R <= 2) ? (a_base | (c0 << 4)) : ((a_base | (c0 << 4)) ^ (j << 4));
-  auto fragments = [&](uint4 (&af)[4], int d) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) af[j] = lds_read_16(a_rd[j], d * kSliceBytes + ((R <= 2) ? j * 16 : 0));
+    for (int j = 0; j < 4; ++j) {
+      af[j] = (R <= 2) ? lds_read_16(base, d * kSliceBytes + j * 16) : lds_read_16(base ^ (j << 4), d * kSliceBytes);
+    }
   };
 
-  // Slot by slot, while the later ones are on their way; the fragments of the next slot are read while this one is
-  // converted (one read at a time right before its MFMA leaves most of the LDS latency in the open).
+  // Slot by slot, while the later ones are on their way.  Up to four rows: the fragments of the next slot are read
+  // while this one is converted (one read at a time right before its MFMA leaves most of the LDS latency in the
+  // open).  More rows: a slot's fragments are there when its weights are, and are read then.
   uint4 af[2][4];
-  fragments(af[0], 0);
+  uint32_t arrived = 0;
+  if constexpr (!kPerSlot) {
+    arrived = zero_once_loaded(w[0][0].x);
+    fragments(af[0], 0, arrived);
+  }
 #pragma unroll
   for (int d = 0; d < D; ++d) {
     __builtin_amdgcn_sched_barrier(0);
-    if (d + 1 < D) fragments(af[(d + 1) & 1], d + 1);
+    if constexpr (kPerSlot) {
+      fragments(af[d & 1], d, zero_once_loaded(w[d][0].x));
+    } else {
+      if (d + 1 < D) fragments(af[(d + 1) & 1], d + 1, arrived);
+    }
     const uint32_t keep = (d < D - 1 || last_ok) ? 0xffffffffu : 0u;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -234,7 +276,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
 #pragma unroll
     for (int x = 0; x < kWaves; ++x) sum += red[x * kPerWave + v];
     const int c = v & 15, r = (v >> 4) & (R - 1), t = v >> (4 + kLgR);
-    const int tile = blockIdx.x * NT + t;
+    const int tile = static_cast<int>(cg) * NT + t;
     if (r < M && tile < tiles) {
       const int col = tile * 16 + c;
       uint32_t h = float_to_bits<BF>(sum);
@@ -258,7 +300,7 @@ int launch_kernel(const blkq4_gemm_args* a) {
   const int slices = a->k / 128;
   const size_t lds = decode_lds_bytes(R, NT, kWaves, D);
   if (a->m > R || slices > kWaves * D || slices <= kWaves * (D - 1) || lds > kMaxLdsBytes || p.lds_bytes != lds ||
-      p.grid != static_cast<uint32_t>((a->n / 16 + NT - 1) / NT)) {
+      p.grid != decode_grid(a->n, NT)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   constexpr auto kernel = decode_mfma_kernel<BS, HAS_ZP, R, NT, kWaves, D>;
@@ -277,9 +319,14 @@ int launch_kernel(const blkq4_gemm_args* a) {
 #define BLKQ4_DECODE_DEPTHS(X, R_, NT_, W_) \
   X(R_, NT_, W_, 1) X(R_, NT_, W_, 2) X(R_, NT_, W_, 3) X(R_, NT_, W_, 4) X(R_, NT_, W_, 5) X(R_, NT_, W_, 6) \
   X(R_, NT_, W_, 7) X(R_, NT_, W_, 8)
+#define BLKQ4_DECODE_DEPTHS_TO_4(X, R_, NT_, W_) X(R_, NT_, W_, 1) X(R_, NT_, W_, 2) X(R_, NT_, W_, 3) X(R_, NT_, W_, 4)
 #define BLKQ4_DECODE_SHAPES(X)                                                                     \
   BLKQ4_DECODE_DEPTHS(X, 1, 1, 4) BLKQ4_DECODE_DEPTHS(X, 1, 1, 8) BLKQ4_DECODE_DEPTHS(X, 1, 1, 16) \
-  BLKQ4_DECODE_DEPTHS(X, 4, 1, 4) BLKQ4_DECODE_DEPTHS(X, 4, 1, 8) BLKQ4_DECODE_DEPTHS(X, 4, 1, 16)
+  BLKQ4_DECODE_DEPTHS(X, 4, 1, 4) BLKQ4_DECODE_DEPTHS(X, 4, 1, 8) BLKQ4_DECODE_DEPTHS(X, 4, 1, 16) \
+  BLKQ4_DECODE_DEPTHS(X, 1, 2, 8) BLKQ4_DECODE_DEPTHS(X, 4, 2, 8)                                  \
+  /* eight rows fit in LDS up to K = 8192, sixteen up to K = 4096 */                               \
+  BLKQ4_DECODE_DEPTHS(X, 8, 1, 8) BLKQ4_DECODE_DEPTHS(X, 8, 2, 8) BLKQ4_DECODE_DEPTHS(X, 8, 3, 8)  \
+  BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 1, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 2, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 3, 8)
 
 template <int BS, bool HAS_ZP>
 int launch_plan(const blkq4_gemm_args* a) {

@@ -1,4 +1,4 @@
-"""The decode kernel (gemmlib_amd/csrc/blkq4_decode.hip: 1 to 4 rows, blocks along K, all of K requested at once),
+"""The decode kernel (gemmlib_amd/csrc/blkq4_decode.hip: 1 to 16 rows, blocks along K, all of K requested at once),
 through blkq4_fp16_gemm_sm80 / blkq4_bf16_gemm_sm80, against the oracle: the reference's exact construction bit
 for bit (test/blkq4_fp16_gemm_sm80_test.cu:194-256,469-472) for every block size, with and without zero-points,
 every number of slices per wave from 1 to 8, slice counts that do not divide among the waves (the last slot of
@@ -28,6 +28,11 @@ EXACT_CASES = [
     (64, False, 1, 1024, 8320),    # 65 slices: 16 waves x 5, one full
     (32, True, 3, 704, 11008), (16, True, 1, 256, 12288), (64, False, 2, 128, 14336), (64, True, 4, 32, 16384),
     (32, False, 1, 128256, 512),   # many workgroups
+    # five to sixteen rows: rows staged slot by slot, 1 to 3 column tiles per workgroup
+    (32, True, 16, 11008, 4096),   # 3 tiles per workgroup, 230 workgroups, the last one with a tile missing
+    (64, False, 8, 4096, 8192), (16, True, 5, 1056, 1152), (32, False, 9, 704, 512), (64, True, 16, 4128, 4096),
+    (16, True, 12, 2080, 2048), (64, True, 7, 32, 1024), (32, True, 16, 128, 128), (16, False, 6, 8192, 6144),
+    (64, False, 13, 8192, 3200), (32, True, 8, 28672, 1024),
 ]
 
 
@@ -67,7 +72,8 @@ def test_exact_on_known_answer_construction_in_bf16(oracle, capi, device, bs, ha
 
 @pytest.mark.parametrize("bs,has_offsets,m,n,k", [
     (64, False, 1, 4096, 4096), (32, True, 4, 11008, 4096), (16, True, 2, 2048, 8192), (64, True, 1, 4096, 11008),
-    (32, False, 3, 14336, 1152), (64, False, 1, 128256, 4096),
+    (32, False, 3, 14336, 1152), (64, False, 1, 128256, 4096), (32, True, 16, 11008, 4096), (16, True, 8, 4096, 8192),
+    (64, True, 11, 5120, 2176),
 ])
 def test_gaussian_within_tolerance_same_bits_every_call(oracle, capi, device, bs, has_offsets, m, n, k):
     a, w = gaussian_problem(5 + m + n + k, m, n, k)
@@ -84,7 +90,7 @@ def test_gaussian_within_tolerance_same_bits_every_call(oracle, capi, device, bs
         assert max_rel_err(got, other) <= 2e-3                           # fp32 sums in another order
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, True, 1, 4096, 4096), (16, True, 4, 2080, 1152)])
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, True, 1, 4096, 4096), (16, True, 4, 2080, 1152), (32, True, 16, 11008, 4096)])
 def test_gaussian_in_bf16(oracle, capi, device, bs, has_offsets, m, n, k):
     a, w = gaussian_bits(oracle, 77 + m + n + k, m, n, k)
     q_w, q_s, q_zp = quantize_bf16(capi, device, bs, w, has_offsets)
@@ -94,7 +100,7 @@ def test_gaussian_in_bf16(oracle, capi, device, bs, has_offsets, m, n, k):
     assert max_rel_err(oracle.bf16_to_f32(got), oracle.bf16_to_f32(ref)) <= 1e-2
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, False, 1, 4096, 4096), (32, True, 3, 1056, 1152), (16, True, 4, 2048, 8192)])
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, False, 1, 4096, 4096), (32, True, 3, 1056, 1152), (16, True, 4, 2048, 8192), (32, True, 16, 11008, 4096)])
 def test_bias_in_the_epilogue_equals_a_separate_add(oracle, capi, device, bs, has_offsets, m, n, k):
     """as the reference module adds it (python/ms_blkq4linear.py:26-27): to the rounded output, in the tensor
     library's way of adding two 16-bit tensors"""
