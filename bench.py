@@ -87,39 +87,39 @@ DESCRIPTION = {
 # figure of a workload is reported only while the library still picks the kernel it was taken from (TRAFFIC_KERNEL).
 COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65552.0, "WRITE_SIZE": 1.0}
 COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
-    "C4": (44108.2, 16387.9),
-    "C2": (4428.6, 8.0),
-    "C3": (13882.7, 344.0),
-    "C5": (860369.0, 229403.7),
-    "C5_prepack": (229443.7, 157730.2),
-    "C4r": (44108.5, 16396.1),
-    "C2r": (4430.1, 8.0),
-    "C1": (866.0, 128.0),
-    "M128": (8649.1, 1024.0),
-    "M256": (24123.1, 11274.1),
-    "M512": (37925.6, 4545.3),
-    "M768N11K": (60847.5, 16513.6),
-    "M256K11K": (43356.1, 19403.8),
-    "V128K": (136363.9, 250.5),
+    "C4": (44108.2, 16384.6),
+    "C2": (4424.1, 8.0),
+    "C3": (13653.7, 344.0),
+    "C5": (860382.2, 229383.4),
+    "C5_prepack": (229443.7, 157730.8),
+    "C4r": (44108.6, 16387.2),
+    "C2r": (4431.1, 8.0),
+    "C1": (875.0, 128.0),
+    "M128": (8661.1, 1024.0),
+    "M256": (24123.1, 11274.0),
+    "M512": (37925.5, 4543.0),
+    "M768N11K": (60847.5, 16512.7),
+    "M256K11K": (43356.1, 19400.7),
+    "V128K": (136348.9, 250.7),
     "B16": (63817.2, 896.0),
-    "C4b": (44128.6, 16392.7),
-    "C2b": (4427.1, 8.0),
+    "C4b": (44128.5, 16386.2),
+    "C2b": (4441.1, 8.0),
 }
 
 
 TRAFFIC_KERNEL = {  # what blkq4_gemm_plan_sm80 said the workload runs when its counters were taken
     "C1": "streaming: 8 waves splitting K, 1 column tile(s) x 32 rows, 2 slices in flight, rows whole in LDS, 2 row group(s), 128 workgroups",
-    "C2": "streaming: 16 waves splitting K, 1 column tile(s) x 16 rows, 2 slices in flight, rows whole in LDS, 1 row group(s), 256 workgroups",
-    "C3": "streaming: 16 waves splitting K, 3 column tile(s) x 16 rows, 2 slices in flight, rows whole in LDS, 1 row group(s), 256 workgroups",
+    "C2": "decode: 4 waves splitting K, 8 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
+    "C3": "decode: 8 waves splitting K, 4 slices requested by each, 3 column tile(s) x 16 row(s), 230 workgroups",
     "C4": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
     "C5": "tile: 256 x 256, 4 + 0 waves, 1792 tiles",
     "C4r": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
     "C2r": "streaming: 16 waves splitting K, 1 column tile(s) x 16 rows, 2 slices in flight, rows whole in LDS, 1 row group(s), 256 workgroups",
     "M128": "streaming: 8 waves splitting K, 4 column tile(s) x 32 rows, 2 slices in flight, rows staged per slice, 4 row group(s), 256 workgroups",
-    "V128K": "streaming: 4 waves with column tiles of their own, 1 column tile(s) x 16 rows, 4 slices in flight, rows whole in LDS, 1 row group(s), 2016 workgroups (walking)",
+    "V128K": "decode: 8 waves splitting K, 4 slices requested by each, 2 column tile(s) x 1 row(s), 4008 workgroups",
     "B16": "streaming: 4 waves splitting K, 4 column tile(s) x 16 rows, 2 slices in flight, rows staged per slice, 1 row group(s), 448 workgroups",
     "C4b": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
-    "C2b": "streaming: 16 waves splitting K, 1 column tile(s) x 16 rows, 2 slices in flight, rows whole in LDS, 1 row group(s), 256 workgroups",
+    "C2b": "decode: 4 waves splitting K, 8 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
     "M256": "tile: 64 x 128, 4 + 4 waves, 128 tiles, the last 128 in 2 parts (workspace 8404992 bytes)",
     "M512": "tile: 64 x 128, 4 + 4 waves, 256 tiles",
     "M768N11K": "tile: 256 x 256, 4 + 0 waves, 129 tiles",

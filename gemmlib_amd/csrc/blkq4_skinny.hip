@@ -329,7 +329,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) BLKQ4_LOAD_SLOT(slot[d], d, cg, ws + kSplit * d, -1, w0, s0, z0);
   }
-  if (A_LDS && kSplit == 1) {
+  if constexpr (A_LDS && kSplit == 1) {
     // everything but the requests of the ring just issued has landed: this wave's share of the rows; then
     // everybody's
     constexpr int kLoads = ROW ? NT * (1 + 4 + (HAS_ZP ? 2 : 0)) : NT * (1 + kMeta * (HAS_ZP ? 2 : 1));
@@ -448,6 +448,9 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
             af[mt][j] = *reinterpret_cast<const uint4*>(ap + mt * 2048 + (((half + j) ^ a_swz) * 16));
           }
       }
+      // all fragment reads are requested before the conversion starts (left to itself the compiler puts each read
+      // right before the MFMA that needs it, which then waits out the whole LDS latency)
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         const uint32_t words[4] = {cur.w[t].x, cur.w[t].y, cur.w[t].z, cur.w[t].w};
