@@ -448,7 +448,7 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
     std::string text;
     if (choice.family == blkq4::kFamilyDecode) {
       const auto& d = choice.d;
-      text = "decode: " + std::to_string(d.waves) + " waves splitting K, " + std::to_string(d.depth) +
+      text = std::string("decode") + (d.row ? " (blocks along N)" : "") + ": " + std::to_string(d.waves) + " waves splitting K, " + std::to_string(d.depth) +
              " slices requested by each, " + std::to_string(d.nt) + " column tile(s) x " + std::to_string(d.rows) +
              " row(s), " + std::to_string((n / 16 + d.nt - 1) / d.nt) + " workgroups";
     } else if (streaming) {

@@ -61,12 +61,12 @@ inline int valu_gemv_waves(int k) {
 inline uint64_t valu_gemv_id(int rows, int waves) {
   return 3ull << 60 | static_cast<uint64_t>(rows) << 8 | static_cast<uint64_t>(waves);
 }
-inline uint64_t decode_id(int rows, int nt, int waves, int depth) {
-  return 4ull << 60 | static_cast<uint64_t>(rows) << 24 | static_cast<uint64_t>(nt) << 16 |
+inline uint64_t decode_id(bool row, int rows, int nt, int waves, int depth) {
+  return 4ull << 60 | static_cast<uint64_t>(row ? 1 : 0) << 32 | static_cast<uint64_t>(rows) << 24 | static_cast<uint64_t>(nt) << 16 |
          static_cast<uint64_t>(waves) << 8 | static_cast<uint64_t>(depth);
 }
 inline uint64_t choice_id(const Choice& c) {
-  if (c.family == kFamilyDecode) return decode_id(c.d.rows, c.d.nt, c.d.waves, c.d.depth);
+  if (c.family == kFamilyDecode) return decode_id(c.d.row != 0, c.d.rows, c.d.nt, c.d.waves, c.d.depth);
   return c.family == kFamilyStreaming
              ? streaming_id(c.s.depth, c.s.nt, c.s.mt, c.s.waves, c.s.am, c.s.split, c.s.refill != 0)
              : tile_id(c.t.rt, c.t.nt, c.t.wm, c.t.wn, c.t.pw, c.t.split_k > 1);
@@ -80,9 +80,11 @@ constexpr int kDecodeMaxRows = 16;
 constexpr int kDecodeMaxDepth = 8;
 
 // LDS of a workgroup: the rows of every wave's slices (256 bytes per row and slice), then the waves' partial
-// tiles (64 bytes per row and tile)
-inline size_t decode_lds_bytes(int rows, int nt, int waves, int depth) {
-  return static_cast<size_t>(waves) * depth * 256 * rows + static_cast<size_t>(waves) * nt * rows * 64;
+// tiles (64 bytes per row and tile), then, with blocks along N, the scales and zero-points of every wave's slices
+// (256 + 128 bytes per slice)
+inline size_t decode_lds_bytes(bool row, int rows, int nt, int waves, int depth) {
+  return static_cast<size_t>(waves) * depth * 256 * rows + static_cast<size_t>(waves) * nt * rows * 64 +
+         (row ? static_cast<size_t>(waves) * depth * 384 : 0);
 }
 
 // Workgroups: one per group of nt column tiles, rounded up to whole sets of 64 groups (the kernel hands eight
@@ -113,9 +115,27 @@ inline uint32_t decode_grid(int n, int nt) {
 // workgroups keep their rows and walk over the column tiles, is faster (M = 16, K = 4096, N = 28672: 17.2 against
 // 20.9 us; M = 8, K = 8192, N = 14336: 15.5 against 18.4; but M = 16, K = 4096, N = 11008: 9.2 against 7.9).
 inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) {
-  if (!column_wise || m < 1 || m > kDecodeMaxRows || (k % 128) != 0 || (n % 16) != 0 ||
+  if (m < 1 || m > kDecodeMaxRows || (k % 128) != 0 || (n % 16) != 0 ||
       static_cast<uint64_t>(k) * static_cast<uint64_t>(n) > (uint64_t{1} << 32)) {
     return false;
+  }
+  if (!column_wise) {
+    // Blocks along N: up to four rows, one column tile per workgroup, eight waves with up to eight slices each
+    // (four waves for short K and for one workgroup per compute unit at most with eight slices each); the scales
+    // and zero-points of a wave's slices, one of each per k, come through LDS.  (M = 1, K = N = 4096: 4.3 against
+    // the streaming kernel's 5.3 us.)
+    const int slices = k / 128;
+    const int tiles = n / 16;
+    if (m > 4 || slices > 8 * kDecodeMaxDepth) return false;
+    const int waves = (slices <= 8 || (slices > 28 && slices <= 32 && tiles <= kComputeUnits)) ? 4 : 8;
+    d->row = 1;
+    d->rows = m == 1 ? 1 : 4;
+    d->nt = 1;
+    d->waves = waves;
+    d->depth = (slices + waves - 1) / waves;
+    d->grid = decode_grid(n, 1);
+    d->lds_bytes = static_cast<uint32_t>(decode_lds_bytes(true, d->rows, 1, waves, d->depth));
+    return true;
   }
   const int slices = k / 128;
   const int tiles = n / 16;
@@ -133,7 +153,7 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
   int nt = 1;
   float best = 0.f;
   for (int t = 1; t <= max_nt; ++t) {
-    if (decode_lds_bytes(rows, t, waves, depth) > kMaxLdsBytes) break;
+    if (decode_lds_bytes(false, rows, t, waves, depth) > kMaxLdsBytes) break;
     const int wgs = (tiles + t - 1) / t;
     float cost = static_cast<float>((wgs + kComputeUnits - 1) / kComputeUnits) * (static_cast<float>(t) + per_workgroup);
     if (rows <= 4 && t == 2 && depth > 4) cost *= 1.1f;
@@ -142,12 +162,13 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
       nt = t;
     }
   }
+  d->row = 0;
   d->rows = rows;
   d->nt = nt;
   d->waves = waves;
   d->depth = depth;
   d->grid = decode_grid(n, nt);
-  d->lds_bytes = static_cast<uint32_t>(decode_lds_bytes(rows, nt, waves, depth));
+  d->lds_bytes = static_cast<uint32_t>(decode_lds_bytes(false, rows, nt, waves, depth));
   if (d->lds_bytes > kMaxLdsBytes) return false;
   if (rows >= 8) {
     const int per_unit = static_cast<size_t>(d->lds_bytes) * 2 <= kMaxLdsBytes ? 2 : 1;  // workgroups a compute unit holds

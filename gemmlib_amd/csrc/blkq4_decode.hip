@@ -69,7 +69,9 @@ constexpr int log2_of(int v) { return v <= 1 ? 0 : 1 + log2_of(v / 2); }
 // R: activation rows kept (a power of two, M <= R <= 16).  NT: 16-column tiles per workgroup that share the
 // activation fragments.  kWaves waves split K; D: slices a wave requests (the last one may be missing).
 // (BF repeats kBF so that the two compilations' kernels carry different names in a trace)
-template <int BS, bool HAS_ZP, int R, int NT, int kWaves, int D, bool BF = kBF>
+// ROW: quantization blocks run along N (one k, BS columns); S and Z are then in the packed order described in
+// blkq4_device.h: a scale and a zero-point per k, the same for the 16 columns of a tile (NT = 1).
+template <int BS, bool HAS_ZP, int R, int NT, int kWaves, int D, bool ROW = false, bool BF = kBF>
 __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t* __restrict__ A,
                                                                 const uint8_t* __restrict__ W,
                                                                 const uint8_t* __restrict__ S,
@@ -83,7 +85,12 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
   constexpr int kSliceBytes = 256 * R;           // a slice's rows in LDS: two pairs of units
   constexpr int kWaveBytes = D * kSliceBytes;    // a wave's rows
   constexpr int kCopies = (kWaveBytes + 1023) / 1024;
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // [wave][kWaveBytes], then the partial tiles
+  // blocks along N: the scales (256 bytes) and zero-points (128 bytes) of a wave's slices, one after the other
+  constexpr int kRowScaleBytes = ROW ? D * 256 : 0;
+  constexpr int kRowMetaBytes = ROW ? D * 384 : 0;
+  static_assert(!ROW || NT == 1, "blocks along N: one column tile per workgroup");
+  // [wave][kWaveBytes] rows, then the partial tiles, then (blocks along N) [wave][kRowMetaBytes]
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   float* red = reinterpret_cast<float*>(smem + kWaves * kWaveBytes);
 
   // The arguments fill the 14 registers that can be preloaded (N and M - 1 share one: N < 2^28, M <= 16), so none
@@ -124,6 +131,25 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
   constexpr bool kPerSlot = R >= 8;
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)(smem)));
   const uint32_t wave_lds = lds0 + wave * kWaveBytes;
+  // Blocks along N: the scales and zero-points of the wave's slices lie in one run each, [K] of the tile's column
+  // block: copied first, 16 bytes per lane (the k range of a missing slot past the end of K fetches the last 16
+  // bytes of the run instead)
+  const uint32_t meta_lds = lds0 + kWaves * kWaveBytes + kWaves * NT * R * 64 + wave * kRowMetaBytes;
+  if constexpr (ROW) {
+    const uint32_t run = (cg * 16 / BS) * static_cast<uint32_t>(K) + static_cast<uint32_t>(s0) * 128u;  // elements
+    const uint32_t run_end = (cg * 16 / BS + 1) * static_cast<uint32_t>(K);
+#pragma unroll
+    for (int c = 0; c * 1024 < kRowScaleBytes; ++c) {
+      const uint32_t off = c * 1024 + lane * 16;
+      if ((c + 1) * 1024 <= kRowScaleBytes || off < static_cast<uint32_t>(kRowScaleBytes)) {
+        async_copy_16(meta_lds + c * 1024, S, min(run + off / 2, run_end - 8) * 2);
+      }
+    }
+    if constexpr (HAS_ZP) {
+      const uint32_t off = lane * 16;  // D * 128 <= 1024 bytes: one copy
+      if (off < static_cast<uint32_t>(D * 128)) async_copy_16(meta_lds + kRowScaleBytes, Z, min(run + off, run_end - 16));
+    }
+  }
 #pragma unroll
   for (int q = 0; q < (kPerSlot ? 0 : kCopies); ++q) {
     const uint32_t off = q * 1024 + lane * 16;
@@ -179,13 +205,15 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
 #pragma unroll
         for (int h = 0; h < kSlotCopies; ++h) async_copy_16(wave_lds + d * kSliceBytes + h * 1024, A, a_off[h] + dd * 256u);
       }
+      if constexpr (!ROW) {
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
+        for (int t = 0; t < NT; ++t) {
 #pragma unroll
-        for (int q = 0; q < kMeta; ++q) {
-          const uint32_t idx = m_idx[t] + dd * m_stride + (q == 0 ? 0u : static_cast<uint32_t>(N));
-          sc[d][t][q] = *reinterpret_cast<const uint16_t*>(S + static_cast<size_t>(idx * 2u));
-          zp[d][t][q] = HAS_ZP ? Z[static_cast<size_t>(idx)] : 8u;
+          for (int q = 0; q < kMeta; ++q) {
+            const uint32_t idx = m_idx[t] + dd * m_stride + (q == 0 ? 0u : static_cast<uint32_t>(N));
+            sc[d][t][q] = *reinterpret_cast<const uint16_t*>(S + static_cast<size_t>(idx * 2u));
+            zp[d][t][q] = HAS_ZP ? Z[static_cast<size_t>(idx)] : 8u;
+          }
         }
       }
 #pragma unroll
@@ -219,15 +247,28 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
     }
   };
 
-  // Slot by slot, while the later ones are on their way.  Up to four rows: the fragments of the next slot are read
-  // while this one is converted (one read at a time right before its MFMA leaves most of the LDS latency in the
-  // open).  More rows: a slot's fragments are there when its weights are, and are read then.
+  // Blocks along N: the 32 scales (64 bytes) and zero-points (32 bytes) of the lane's unit, from the wave's copy
+  auto row_meta = [&](uint4 (&rs)[4], uint4 (&rz)[2], int d, uint32_t arrived) {
+    const uint32_t base = meta_lds + g * 64 + arrived;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) rs[q] = lds_read_16(base, d * 256 + q * 16);
+    if constexpr (HAS_ZP) {
+      const uint32_t zbase = meta_lds + kRowScaleBytes + g * 32 + arrived;
+#pragma unroll
+      for (int q = 0; q < 2; ++q) rz[q] = lds_read_16(zbase, d * 128 + q * 16);
+    }
+  };
+
+  // Slot by slot, while the later ones are on their way.  Up to four rows: the fragments of the next slot (and its
+  // scales and zero-points, with blocks along N) are read while this one is converted (one read at a time right
+  // before its MFMA leaves most of the LDS latency in the open).  More rows: a slot's fragments are there when its
+  // weights are, and are read then.
   uint4 af[2][4];
+  uint4 rs[2][4], rz[2][2];
   uint32_t arrived = 0;
-  if constexpr (!kPerSlot) {
-    arrived = zero_once_loaded(w[0][0].x);
-    fragments(af[0], 0, arrived);
-  }
+  if constexpr (!kPerSlot || ROW) arrived = zero_once_loaded(w[0][0].x);
+  if constexpr (!kPerSlot) fragments(af[0], 0, arrived);
+  if constexpr (ROW) row_meta(rs[0], rz[0], 0, arrived);
 #pragma unroll
   for (int d = 0; d < D; ++d) {
     __builtin_amdgcn_sched_barrier(0);
@@ -236,6 +277,9 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
     } else {
       if (d + 1 < D) fragments(af[(d + 1) & 1], d + 1, arrived);
     }
+    if constexpr (ROW) {
+      if (d + 1 < D) row_meta(rs[(d + 1) & 1], rz[(d + 1) & 1], d + 1, arrived);
+    }
     const uint32_t keep = (d < D - 1 || last_ok) ? 0xffffffffu : 0u;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -243,7 +287,39 @@ __global__ __launch_bounds__(64 * kWaves) void decode_mfma_kernel(const uint8_t*
       for (int t = 0; t < NT; ++t) {
         const uint32_t word = vec_word(w[d][t], j);
         const int q = (kMeta == 2) ? (j >> 1) : 0;
-        if constexpr (BF) {
+        if constexpr (ROW) {
+          // word j is rows 8 hh .. 8 hh + 7 of 16-row group j / 2 of the unit: pair i has its scales in 32-bit word
+          // 2 i + hh of the group and its zero-points in byte pair hh of word i (blkq4_skinny.hip has the same)
+          const int hh = j & 1;
+          const uint4 s0v = rs[d & 1][2 * (j >> 1)], s1v = rs[d & 1][2 * (j >> 1) + 1];
+          const uint32_t sw[8] = {s0v.x, s0v.y, s0v.z, s0v.w, s1v.x, s1v.y, s1v.z, s1v.w};
+          const uint4 zq = HAS_ZP ? rz[d & 1][j >> 1] : make_uint4(0, 0, 0, 0);
+          const uint32_t zw[4] = {zq.x, zq.y, zq.z, zq.w};
+          const uint32_t y = word >> 8;
+          half2_t p[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const uint32_t zpair = HAS_ZP ? ((zw[i] >> (8 * hh)) & 0x00ff00ffu) : 0x00080008u;
+            const uint32_t src = (i >= 2) ? y : word;
+            // q - zp of the pair, exact
+            const half2_t dq = ((i & 1) == 0)
+                ? as_half2((src & masks.lo_mask) | masks.magic_1024) + as_half2(0xE400E400u | zpair)
+                : as_half2((src & masks.hi_mask) | masks.magic_64) + as_half2(0xD400D400u | (zpair << 4));
+            if constexpr (BF) {
+              p[i] = as_half2(row_pair_bf16(dq, sw[2 * i + hh] & keep));  // a bf16 pair in the same register
+            } else {
+              p[i] = dq * as_half2(sw[2 * i + hh] & keep);
+            }
+          }
+          half8_t wf;
+          wf[0] = p[0][0]; wf[1] = p[0][1]; wf[2] = p[1][0]; wf[3] = p[1][1];
+          wf[4] = p[2][0]; wf[5] = p[2][1]; wf[6] = p[3][0]; wf[7] = p[3][1];
+          if constexpr (BF) {
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf), as_bf16x8(af[d & 1][j]), acc[t], 0, 0, 0);
+          } else {
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, as_half8(af[d & 1][j]), acc[t], 0, 0, 0);
+          }
+        } else if constexpr (BF) {
           const Bf16Consts bc = make_bf16_consts(sc[d][t][q] & keep, zp[d][t][q]);
           const bf16x8_t wf = dequant_word_bf16(word, bc, masks);
           acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, as_bf16x8(af[d & 1][j]), acc[t], 0, 0, 0);
@@ -292,18 +368,18 @@ hipError_t raise_lds_limit() {
 }
 
 // One instantiation with the geometry of the plan (blkq4_choose.h).  What the kernel assumes is checked here.
-template <int BS, bool HAS_ZP, int R, int NT, int kWaves, int D>
+template <int BS, bool HAS_ZP, bool ROW, int R, int NT, int kWaves, int D>
 int launch_kernel(const blkq4_gemm_args* a) {
   const blkq4_decode_plan& p = a->decode;
-  if (a->launched_id != nullptr) *a->launched_id = decode_id(R, NT, kWaves, D);
+  if (a->launched_id != nullptr) *a->launched_id = decode_id(ROW, R, NT, kWaves, D);
   if (a->dry_run) return 0;
   const int slices = a->k / 128;
-  const size_t lds = decode_lds_bytes(R, NT, kWaves, D);
+  const size_t lds = decode_lds_bytes(ROW, R, NT, kWaves, D);
   if (a->m > R || slices > kWaves * D || slices <= kWaves * (D - 1) || lds > kMaxLdsBytes || p.lds_bytes != lds ||
       p.grid != decode_grid(a->n, NT)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
-  constexpr auto kernel = decode_mfma_kernel<BS, HAS_ZP, R, NT, kWaves, D>;
+  constexpr auto kernel = decode_mfma_kernel<BS, HAS_ZP, R, NT, kWaves, D, ROW>;
   if (lds > 64 * 1024) {
     if (hipError_t e = raise_lds_limit<kernel>(); e != hipSuccess) return static_cast<int>(e);
   }
@@ -327,29 +403,45 @@ int launch_kernel(const blkq4_gemm_args* a) {
   /* eight rows fit in LDS up to K = 8192, sixteen up to K = 4096 */                               \
   BLKQ4_DECODE_DEPTHS(X, 8, 1, 8) BLKQ4_DECODE_DEPTHS(X, 8, 2, 8) BLKQ4_DECODE_DEPTHS(X, 8, 3, 8)  \
   BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 1, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 2, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 3, 8)
+// blocks along N: up to four rows, one tile, K up to 8192
+#define BLKQ4_DECODE_ROW_SHAPES(X)                                                    \
+  BLKQ4_DECODE_DEPTHS(X, 1, 1, 8) BLKQ4_DECODE_DEPTHS(X, 4, 1, 8)                     \
+  X(1, 1, 4, 1) X(1, 1, 4, 2) X(1, 1, 4, 8) X(4, 1, 4, 1) X(4, 1, 4, 2) X(4, 1, 4, 8)
 
-template <int BS, bool HAS_ZP>
+template <int BS, bool HAS_ZP, bool ROW>
 int launch_plan(const blkq4_gemm_args* a) {
   const blkq4_decode_plan& p = a->decode;
 #define BLKQ4_TRY(R_, NT_, W_, D_) \
-  if (p.rows == R_ && p.nt == NT_ && p.waves == W_ && p.depth == D_) return launch_kernel<BS, HAS_ZP, R_, NT_, W_, D_>(a);
-  BLKQ4_DECODE_SHAPES(BLKQ4_TRY)
+  if (p.rows == R_ && p.nt == NT_ && p.waves == W_ && p.depth == D_) return launch_kernel<BS, HAS_ZP, ROW, R_, NT_, W_, D_>(a);
+  if constexpr (ROW) {
+    BLKQ4_DECODE_ROW_SHAPES(BLKQ4_TRY)
+  } else {
+    BLKQ4_DECODE_SHAPES(BLKQ4_TRY)
+  }
 #undef BLKQ4_TRY
   return static_cast<int>(hipErrorInvalidValue);  // a shape that does not exist
 }
 
 template <int BS>
 int launch_bs(const blkq4_gemm_args* a) {
-  return a->zero_points ? launch_plan<BS, true>(a) : launch_plan<BS, false>(a);
+  if (a->column_wise) return a->zero_points ? launch_plan<BS, true, false>(a) : launch_plan<BS, false, false>(a);
+  return a->zero_points ? launch_plan<BS, true, true>(a) : launch_plan<BS, false, true>(a);
 }
 
 }  // namespace
 
 extern "C" int BLKQ4_DECODE_ENTRY(const blkq4_gemm_args* a) {
   // 32-bit offsets: the packed weights end below 4 GiB
-  if (a->m < 1 || a->m > 16 || !a->column_wise || (a->n % 16) != 0 || (a->k % 128) != 0 ||
+  if (a->m < 1 || a->m > 16 || (a->n % 16) != 0 || (a->k % 128) != 0 ||
       static_cast<uint64_t>(a->k) * static_cast<uint64_t>(a->n) > (uint64_t{1} << 32)) {
     return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (!a->column_wise) {
+    // blocks along N: a 16-column tile lies inside one block, and the meta data are copied 16 bytes at a time
+    if ((a->n % a->block_size) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 15u) != 0 ||
+        (reinterpret_cast<uintptr_t>(a->zero_points) & 15u) != 0) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
   }
   switch (a->block_size) {
     case 16: return launch_bs<16>(a);

@@ -74,6 +74,7 @@ typedef struct {
  * tiles per workgroup, `waves` waves that split K, `depth` slices requested by each.  Filled in by
  * blkq4::decode_shape() (blkq4_choose.h). */
 typedef struct {
+  int row;             /* 1: blocks along N */
   int rows, nt, waves, depth;
   uint32_t grid;       /* workgroups */
   uint32_t lds_bytes;  /* dynamic LDS */

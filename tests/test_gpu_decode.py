@@ -36,12 +36,58 @@ EXACT_CASES = [
 ]
 
 
-def _run(capi, device, bs, a, q_w, q_s, q_zp, n, **kw):
+# blocks along N (up to four rows): 4 and 8 waves, 1 to 8 slices each, waves with an empty slot or none at all
+ROW_CASES = [
+    (64, False, 1, 4096, 4096), (64, True, 1, 1024, 1024), (32, True, 2, 96, 128), (16, True, 3, 160, 256),
+    (32, False, 4, 2080, 384), (64, True, 1, 4160, 2048), (16, False, 1, 704, 3200), (32, True, 4, 1056, 5120),
+    (64, False, 2, 1024, 8192), (16, True, 1, 32000, 1152), (64, True, 3, 128, 640), (32, True, 1, 14336, 4096),
+]
+
+
+def _run(capi, device, bs, a, q_w, q_s, q_zp, n, col=True, **kw):
     m, k = a.shape
     out = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
-    capi.gemm(bs, True, m, n, k, to_dev(a, device), q_w, q_s, q_zp, out, **kw)
+    capi.gemm(bs, col, m, n, k, to_dev(a, device), q_w, q_s, q_zp, out, **kw)
     torch.cuda.synchronize()
     return to_np(out)
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", ROW_CASES)
+def test_blocks_along_n_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
+    """the reference's row-wise construction (test/blkq4_fp16_gemm_sm80_test.cu:480-499), fp16 and bf16"""
+    assert capi.gemm_plan(bs, False, m, n, k, has_offsets)[2].startswith("decode (blocks along N):")
+    rng = np.random.default_rng(m * 131 + n * 17 + k + bs + has_offsets)
+    kat = oracle.kat_generate(bs, False, k, n, has_offsets)
+    a = grid_activations(rng, m, k)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, kat["weights"], has_offsets, column_wise=False)
+    ref = oracle.gemm(a, kat["weights"])
+    got = _run(capi, device, bs, a, q_w, q_s, q_zp, n, col=False)
+    if not np.array_equal(got.view(np.uint16), ref.view(np.uint16)):
+        bad = np.argwhere(got.view(np.uint16) != ref.view(np.uint16))
+        raise AssertionError(f"{bad.shape[0]} of {m * n} outputs differ, first {bad[:5].tolist()}")
+    if n <= 8192:
+        katb = bf16_kat(oracle, bs, k, n, has_offsets, seed=m + n + k, column_wise=False)
+        ab = grid_activations_bf16(oracle, rng, m, k)
+        q_w, q_s, q_zp = quantize_bf16(capi, device, bs, katb["weights"], has_offsets, col=False)
+        assert np.array_equal(gemm_bf16(capi, device, bs, ab, q_w, q_s, q_zp, n, col=False), oracle.gemm(ab, katb["weights"], bf16=True))
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, False, 1, 4096, 4096), (32, True, 4, 2816, 1152), (16, True, 2, 2048, 8192)])
+def test_blocks_along_n_gaussian_and_bias(oracle, capi, device, bs, has_offsets, m, n, k):
+    a, w = gaussian_problem(9 + m + n + k, m, n, k)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, w, has_offsets, column_wise=False)
+    canon, s, z = oracle.quantize(bs, False, w, has_offsets)
+    ref = oracle.gemm(a, oracle.dequantize(bs, False, canon, s, z))
+    got = _run(capi, device, bs, a, q_w, q_s, q_zp, n, col=False)
+    assert max_rel_err(got, ref) <= 1e-2
+    again = _run(capi, device, bs, a, q_w, q_s, q_zp, n, col=False)
+    assert np.array_equal(again.view(np.uint16), got.view(np.uint16))
+    g = torch.Generator(device="cpu").manual_seed(n)
+    bias = (torch.randn(n, generator=g) * 0.5).to(torch.float16).to(device)
+    plain = torch.from_numpy(got.view(np.int16)).to(device).view(torch.float16)
+    fused = _run(capi, device, bs, a, q_w, q_s, q_zp, n, col=False, bias=bias)
+    plain += bias
+    assert np.array_equal(fused.view(np.uint16), to_np(plain).view(np.uint16))
 
 
 @pytest.mark.parametrize("bs,has_offsets,m,n,k", EXACT_CASES)
