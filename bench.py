@@ -88,22 +88,22 @@ DESCRIPTION = {
 COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65552.0, "WRITE_SIZE": 1.0}
 COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
     "C4": (44108.2, 16384.6),
-    "C2": (4424.1, 8.0),
-    "C3": (13653.7, 344.0),
-    "C5": (860382.2, 229383.4),
-    "C5_prepack": (229443.7, 157730.8),
-    "C4r": (44108.6, 16387.2),
+    "C2": (4428.1, 8.0),
+    "C3": (13653.6, 344.0),
+    "C5": (860404.6, 229384.7),
+    "C5_prepack": (229443.8, 157731.3),
+    "C4r": (44108.6, 16387.8),
     "C2r": (4431.1, 8.0),
     "C1": (875.0, 128.0),
     "M128": (8661.1, 1024.0),
-    "M256": (24123.1, 11274.0),
-    "M512": (37925.5, 4543.0),
+    "M256": (24123.1, 11274.2),
+    "M512": (37925.5, 4542.0),
     "M768N11K": (60847.5, 16512.7),
-    "M256K11K": (43356.1, 19400.7),
-    "V128K": (136348.9, 250.7),
+    "M256K11K": (43356.1, 19401.4),
+    "V128K": (136348.9, 252.3),
     "B16": (63817.2, 896.0),
-    "C4b": (44128.5, 16386.2),
-    "C2b": (4441.1, 8.0),
+    "C4b": (44128.5, 16386.3),
+    "C2b": (4440.1, 8.0),
 }
 
 
@@ -114,7 +114,7 @@ TRAFFIC_KERNEL = {  # what blkq4_gemm_plan_sm80 said the workload runs when its 
     "C4": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
     "C5": "tile: 256 x 256, 4 + 0 waves, 1792 tiles",
     "C4r": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
-    "C2r": "streaming: 16 waves splitting K, 1 column tile(s) x 16 rows, 2 slices in flight, rows whole in LDS, 1 row group(s), 256 workgroups",
+    "C2r": "decode (blocks along N): 4 waves splitting K, 8 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
     "M128": "streaming: 8 waves splitting K, 4 column tile(s) x 32 rows, 2 slices in flight, rows staged per slice, 4 row group(s), 256 workgroups",
     "V128K": "decode: 8 waves splitting K, 4 slices requested by each, 2 column tile(s) x 1 row(s), 4008 workgroups",
     "B16": "streaming: 4 waves splitting K, 4 column tile(s) x 16 rows, 2 slices in flight, rows staged per slice, 1 row group(s), 448 workgroups",
