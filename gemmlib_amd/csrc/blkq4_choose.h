@@ -12,6 +12,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <initializer_list>
+
 #include "blkq4_device.h"
 
 namespace blkq4 {
@@ -271,15 +273,26 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
   };
   s.row_groups = 1;
   if (m > 16) {
-    // Row groups of 32 rows (two row tiles share one conversion of the weights), eight waves.  Every workgroup
-    // fetches the 32 rows of its group for all of K, so wide workgroups (more column tiles) mean less
-    // activation traffic; but there should be a workgroup for most compute units (measured: four tiles per
-    // workgroup from 160 workgroups of four on, two from 160 of two on).  Blocks along N: 28 registers of
+    // Row groups of 32 rows (two row tiles share one conversion of the weights), eight waves.  A workgroup's time
+    // grows with its column tiles -- measured at K = 4096: 3.0 + 1.73 us per tile (M = 128, N = 4096 with 4, 6 and 8
+    // tiles: 11.6, 15.2, 18.5 us; with 2, in two rounds: 14.9) -- and the busiest compute unit works through
+    // ceil(workgroups / 256) of them: as many tiles per workgroup (1, 2, 4, 6, 8) as make that product smallest
+    // (M = 64, N = 11008: 344 workgroups of four tiles 21.8 us, 230 of six 15.9).  Blocks along N: 28 registers of
     // packed weights, scales and zero-points per slot and tile, so one tile.
     s.row_groups = (m + 31) / 32;
     s.rows_log2 = 5;
-    const long tiles = static_cast<long>(n / 16) * s.row_groups;
-    const int nt = row ? 1 : tiles >= 640 ? 4 : tiles >= 320 ? 2 : 1;
+    int nt = 1;
+    if (!row) {
+      double best = 0.0;
+      for (const int t : {1, 2, 4, 6, 8}) {
+        const long wgs = static_cast<long>(s.row_groups) * ((n / 16 + t - 1) / t);
+        const double cost = static_cast<double>((wgs + kComputeUnits - 1) / kComputeUnits) * (3.0 + 1.73 * t);
+        if (t == 1 || cost < best) {
+          best = cost;
+          nt = t;
+        }
+      }
+    }
     const bool rows_fit = static_cast<size_t>(k) * 2 * 32 <= kMaxLdsBytes;
     set(2, nt, 2, 8, rows_fit ? kRowsWholeInLds : kRowsPerSlotInLds, 8);
     streaming_geometry(&s, row, n, k);

@@ -630,8 +630,10 @@ int launch_kernel(const blkq4_gemm_args* a) {
 #define BLKQ4_P kRowsPerSlotInLds
 #define BLKQ4_STREAMING_SHAPES(X)                                                                          \
   /* row groups of 32 */                                                                                   \
-  X(2, 1, 2, 8, BLKQ4_W, 8) X(2, 2, 2, 8, BLKQ4_W, 8) X(2, 4, 2, 8, BLKQ4_W, 8)                            \
-  X(2, 1, 2, 8, BLKQ4_P, 8) X(2, 2, 2, 8, BLKQ4_P, 8) X(2, 4, 2, 8, BLKQ4_P, 8)                            \
+  X(2, 1, 2, 8, BLKQ4_W, 8) X(2, 2, 2, 8, BLKQ4_W, 8) X(2, 4, 2, 8, BLKQ4_W, 8) X(2, 6, 2, 8, BLKQ4_W, 8)  \
+  X(2, 8, 2, 8, BLKQ4_W, 8)                                                                                \
+  X(2, 1, 2, 8, BLKQ4_P, 8) X(2, 2, 2, 8, BLKQ4_P, 8) X(2, 4, 2, 8, BLKQ4_P, 8) X(2, 6, 2, 8, BLKQ4_P, 8)  \
+  X(2, 8, 2, 8, BLKQ4_P, 8)                                                                                \
   /* waves with column tiles of their own */                                                               \
   X(4, 1, 1, 4, BLKQ4_W, 1)                                                                                \
   /* wide layers, rows staged per slice */                                                                 \

@@ -100,7 +100,15 @@ VERY_WIDE_CASES = [
 ]
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + SMALL_TILE_CASES + WIDE_TILE32_CASES + LONG_K_CASES + VERY_WIDE_CASES)
+# row groups of 32 with six and eight column tiles per workgroup (rows whole in LDS and staged per slice), the last
+# workgroup of a row group with tiles missing
+SIX_AND_EIGHT_TILE_CASES = [
+    (64, True, 48, 11008, 1152), (32, False, 64, 11008, 4096), (16, True, 96, 8192, 640), (64, True, 100, 8224, 4096),
+    (32, True, 33, 11040, 2176), (64, False, 60, 14336, 4160),
+]
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + SMALL_TILE_CASES + WIDE_TILE32_CASES + LONG_K_CASES + VERY_WIDE_CASES + SIX_AND_EIGHT_TILE_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
 
