@@ -80,6 +80,7 @@ inline uint64_t choice_id(const Choice& c) {
 
 constexpr int kDecodeMaxRows = 16;
 constexpr int kDecodeMaxDepth = 8;
+constexpr int kDecodeMaxDepthSixteenWaves = 14;  // up to four rows: K up to 28672
 
 // LDS of a workgroup: the rows of every wave's slices (256 bytes per row and slice), then the waves' partial
 // tiles (64 bytes per row and tile), then, with blocks along N, the scales and zero-points of every wave's slices
@@ -146,10 +147,10 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
   if (rows <= 4) {
     if (slices <= 8 || (slices > 24 && slices <= 32 && tiles <= kComputeUnits)) waves = 4;
     if (slices > 8 * kDecodeMaxDepth) waves = 16;
-    if (slices > 16 * kDecodeMaxDepth) return false;
+    if (slices > 16 * kDecodeMaxDepthSixteenWaves) return false;
   }
   const int depth = (slices + waves - 1) / waves;
-  if (depth > ((rows == 16) ? 4 : kDecodeMaxDepth)) return false;
+  if (depth > ((rows == 16) ? 4 : (rows <= 4 && waves == 16) ? kDecodeMaxDepthSixteenWaves : kDecodeMaxDepth)) return false;
   const int max_nt = rows >= 8 ? 3 : (waves == 8 ? 2 : 1);  // the instantiations that exist
   const float per_workgroup = rows == 1 ? 0.1f : 0.5f;
   int nt = 1;

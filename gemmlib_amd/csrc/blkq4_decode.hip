@@ -1,6 +1,6 @@
-// Decode kernel for gfx950: GEMV and GEMM with up to 16 activation rows, blocks along K, when a workgroup can
-// request all of K at once.  The same arithmetic as the weight-streaming kernel (blkq4_skinny.hip), with as few
-// instructions around it as the job allows.
+// Decode kernel for gfx950: GEMV and GEMM with up to 16 activation rows and blocks along K (up to four rows with
+// blocks along N), when a workgroup can request all of K at once.  The same arithmetic as the weight-streaming
+// kernel (blkq4_skinny.hip), with as few instructions around it as the job allows.
 //
 // A compute unit issues one instruction per wave every four cycles, and the waves of a SIMD share one issue slot
 // per instruction type, so at these sizes (a few microseconds, tens of kilobytes of weights per compute unit)
@@ -24,7 +24,10 @@
 //     first weights and need no barrier;
 //   - one barrier: the waves' partial tiles meet in LDS and are summed in the order of the waves;
 //   - neighbouring column tiles run on the same XCD at about the same time and share the cache lines of their
-//     scales and zero-points (16 columns use 32 and 16 bytes of a row).
+//     scales and zero-points (16 columns use 32 and 16 bytes of a row);
+//   - blocks along N: a lane's 32 weights have a scale and a zero-point each, the same for the 16 columns of the
+//     tile; a wave's slices have them in one contiguous run, which two or three copy instructions bring to LDS
+//     (the streaming kernel fetches them with six loads per slot and lane).
 // Dequantization is the streaming kernel's (blkq4_dequant.h: one rounding per weight), accumulation fp32 in
 // v_mfma_f32_16x16x32_{f16,bf16} with the weights as the row operand.
 
@@ -396,10 +399,14 @@ int launch_kernel(const blkq4_gemm_args* a) {
   X(R_, NT_, W_, 1) X(R_, NT_, W_, 2) X(R_, NT_, W_, 3) X(R_, NT_, W_, 4) X(R_, NT_, W_, 5) X(R_, NT_, W_, 6) \
   X(R_, NT_, W_, 7) X(R_, NT_, W_, 8)
 #define BLKQ4_DECODE_DEPTHS_TO_4(X, R_, NT_, W_) X(R_, NT_, W_, 1) X(R_, NT_, W_, 2) X(R_, NT_, W_, 3) X(R_, NT_, W_, 4)
+#define BLKQ4_DECODE_DEPTHS_9_TO_14(X, R_, NT_, W_) \
+  X(R_, NT_, W_, 9) X(R_, NT_, W_, 10) X(R_, NT_, W_, 11) X(R_, NT_, W_, 12) X(R_, NT_, W_, 13) X(R_, NT_, W_, 14)
 #define BLKQ4_DECODE_SHAPES(X)                                                                     \
   BLKQ4_DECODE_DEPTHS(X, 1, 1, 4) BLKQ4_DECODE_DEPTHS(X, 1, 1, 8) BLKQ4_DECODE_DEPTHS(X, 1, 1, 16) \
   BLKQ4_DECODE_DEPTHS(X, 4, 1, 4) BLKQ4_DECODE_DEPTHS(X, 4, 1, 8) BLKQ4_DECODE_DEPTHS(X, 4, 1, 16) \
   BLKQ4_DECODE_DEPTHS(X, 1, 2, 8) BLKQ4_DECODE_DEPTHS(X, 4, 2, 8)                                  \
+  /* K up to 28672 with sixteen waves */                                                           \
+  BLKQ4_DECODE_DEPTHS_9_TO_14(X, 1, 1, 16) BLKQ4_DECODE_DEPTHS_9_TO_14(X, 4, 1, 16)                \
   /* eight rows fit in LDS up to K = 8192, sixteen up to K = 4096 */                               \
   BLKQ4_DECODE_DEPTHS(X, 8, 1, 8) BLKQ4_DECODE_DEPTHS(X, 8, 2, 8) BLKQ4_DECODE_DEPTHS(X, 8, 3, 8)  \
   BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 1, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 2, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 3, 8)

@@ -28,6 +28,7 @@ EXACT_CASES = [
     (64, False, 1, 1024, 8320),    # 65 slices: 16 waves x 5, one full
     (32, True, 3, 704, 11008), (16, True, 1, 256, 12288), (64, False, 2, 128, 14336), (64, True, 4, 32, 16384),
     (32, False, 1, 128256, 512),   # many workgroups
+    (64, False, 1, 256, 28672), (32, True, 4, 128, 18432), (16, True, 2, 64, 17408),   # sixteen waves x 14, 9, 9 (uneven)
     # five to sixteen rows: rows staged slot by slot, 1 to 3 column tiles per workgroup
     (32, True, 16, 11008, 4096),   # 3 tiles per workgroup, 230 workgroups, the last one with a tile missing
     (64, False, 8, 4096, 8192), (16, True, 5, 1056, 1152), (32, False, 9, 704, 512), (64, True, 16, 4128, 4096),
