@@ -498,6 +498,12 @@ def bench_context(torch, capi, device, head_problem, steps, warmup):
                     for w, sc in zip(ws, ss)]
         wall, evt, _ = timed_region(torch, launches, floor_launches, warmup)
         out["c2_requests_only_us" if with_scales else "c2_weight_requests_only_us"] = round(evt / floor_launches * 1e6, 3)
+    # the same bytes requested the way the decode kernel requests them (four waves, eight slices each, at once)
+    probe.blkq4_probe_decode_requests.argtypes = probe.blkq4_probe_stream.argtypes
+    launches = [(lambda w=w, sc=sc: probe.blkq4_probe_decode_requests(w.data_ptr(), sc.data_ptr(), n, k, scratch.data_ptr(), stream_ptr()))
+                for w, sc in zip(ws, ss)]
+    wall, evt, _ = timed_region(torch, launches, floor_launches, warmup)
+    out["c2_decode_requests_only_us"] = round(evt / floor_launches * 1e6, 3)
     del ws, ss
     out["gemv_forms_c2_shape"] = bench_gemv_forms(torch, capi, device, [(1, 4096, 4096, 64, False)], steps)[0]
     if head_problem is not None:

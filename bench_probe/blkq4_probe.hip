@@ -39,6 +39,28 @@ __global__ __launch_bounds__(64 * WAVES) void stream_kernel(const uint4* __restr
   if (a == 0x12345678u) out[blockIdx.x] = a;  // keeps the loads alive, (almost) never stores
 }
 
+// The decode kernel's requests for M = 1, blocks of 64 along K: a workgroup of WAVES waves owns 16 columns, wave w
+// the D consecutive slices from w D on, all requested at once with 32-bit offsets (scale first, then the unit).
+template <int WAVES, int D>
+__global__ __launch_bounds__(64 * WAVES) void decode_requests_kernel(const uint8_t* __restrict__ W,
+                                                                     const uint8_t* __restrict__ S, unsigned* out,
+                                                                     int N) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nl = lane & 15, g = lane >> 4;
+  const unsigned unit0 = 4u * (wave * D) + g;
+  const unsigned col = blockIdx.x * 16 + nl;
+  uint4 v[D];
+  unsigned sc[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    sc[d] = *reinterpret_cast<const uint16_t*>(S + (((unit0 >> 1) + 2u * d) * N + col) * 2u);
+    v[d] = *reinterpret_cast<const uint4*>(W + ((unit0 + 4u * d) * N + col) * 16u);
+  }
+  unsigned a = 0;
+#pragma unroll
+  for (int d = 0; d < D; ++d) a ^= v[d].x ^ v[d].y ^ v[d].z ^ v[d].w ^ sc[d];
+  if (a == 0x12345678u) out[blockIdx.x] = a;  // keeps the loads alive, (almost) never stores
+}
+
 typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
 typedef float probe_float16 __attribute__((ext_vector_type(16)));
 
@@ -126,6 +148,16 @@ PROBE_EXPORT int blkq4_probe_stream16(const void* packed_w, const void* scales, 
                        static_cast<const uint4*>(packed_w), static_cast<const uint16_t*>(nullptr),
                        static_cast<unsigned*>(scratch), n, k);
   }
+  return static_cast<int>(hipGetLastError());
+}
+
+// the decode kernel's requests: four waves with eight slices each (k = 4096)
+PROBE_EXPORT int blkq4_probe_decode_requests(const void* packed_w, const void* scales, int n, int k, void* scratch,
+                                             void* stream) {
+  if (n % 16 != 0 || k != 4096) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL((decode_requests_kernel<4, 8>), dim3(n / 16), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint8_t*>(packed_w), static_cast<const uint8_t*>(scales),
+                     static_cast<unsigned*>(scratch), n);
   return static_cast<int>(hipGetLastError());
 }
 
