@@ -333,12 +333,39 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
     // unit: eight waves from 832 column tiles on, four from 1536 on.  Measured against every other shape of
     // workgroup: M = 16, K = 8192: N = 14336 24.3 -> 17.6 us, N = 28672 43.1 -> 34.1 us; rows that would fit
     // (M = 16, K = 4096, N = 14336: 13.2 -> 11.1 us) gain less or nothing, never lose more than 3 %.
-    if (tiles >= 1536) {
-      set(2, 4, 1, 4, kRowsPerSlotInLds, 4);
-      return done();
-    }
+    //
+    // Tiles per workgroup and waves: every workgroup is resident from the start (no second round, no walking), and
+    // the launch takes as long as the busiest compute unit, which has ceil(workgroups / 256) workgroups of nt
+    // tiles each; a unit with four waves only hides a twelfth less of the latency, one with eight a fifteenth
+    // (M = 16, K = 8192: N = 28672, 448 workgroups of four tiles and four waves 30.2 us, 256 of seven tiles and
+    // eight waves 28.5, and four waves 29.6; N = 57344, 896 of four tiles 60.9, 512 of seven 52.1; N = 14336, 224
+    // of four tiles and eight waves 17.3, and four waves 19.7, 128 of seven tiles 24.4).  Four tiles (four waves
+    // from 1536 column tiles on, else eight) unless another shape promises 3 % less.
     if (tiles >= 832) {
-      set(2, 4, 1, 8, kRowsPerSlotInLds, 8);
+      const size_t red_rows = size_t{1} << s.rows_log2;
+      auto busiest = [&](int nt, int waves, bool all_resident) -> double {
+        const size_t lds = static_cast<size_t>(waves) * 2 * 4096 + static_cast<size_t>(waves) * nt * red_rows * 64;
+        const long by_lds = static_cast<long>(kMaxLdsBytes / lds), by_waves = 32 / waves;
+        const long resident = by_lds < by_waves ? by_lds : by_waves;
+        const long per_unit = ((tiles + nt - 1) / nt + kComputeUnits - 1) / kComputeUnits;
+        if (all_resident && per_unit > resident) return -1.0;
+        const long on_unit = per_unit * waves;
+        return static_cast<double>(per_unit * nt) * (on_unit <= 4 ? 1.12 : on_unit <= 8 ? 1.07 : 1.0);
+      };
+      int nt = 4, waves = tiles >= 1536 ? 4 : 8;
+      const double usual = busiest(nt, waves, false);
+      double best = usual;
+      for (const int w : {8, 4}) {
+        for (const int t : {5, 6, 7}) {
+          const double cost = busiest(t, w, true);
+          if (cost > 0.0 && cost < best && cost < 0.97 * usual) {
+            best = cost;
+            nt = t;
+            waves = w;
+          }
+        }
+      }
+      set(2, nt, 1, waves, kRowsPerSlotInLds, waves);
       return done();
     }
   }
@@ -496,7 +523,11 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
 // it is expected to be faster than the tile kernel, whose grid cannot fill the chip when m is small.
 // The streaming kernel's time grows with row groups x n x k (2.8 us per row group at n = k = 4096) and, once
 // it has more workgroups than compute units, with whole rounds of them.
+constexpr uint64_t kStreamingMaxWeights = uint64_t{1} << 33;
+
 inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const StreamingShape& s, double tile_us) {
+  // its offsets into the packed weights (K N / 2 bytes) are 32 bits wide
+  if (static_cast<uint64_t>(k) * static_cast<uint64_t>(n) > kStreamingMaxWeights) return false;
   if (m <= 16) return true;
   if (m <= 32) {
     // 17 to 32 rows: the streaming kernel wins unless it cannot keep the rows in LDS for all of K (it then

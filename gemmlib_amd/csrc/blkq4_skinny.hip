@@ -267,24 +267,39 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   // a slot past the end asks for valid units (so every slot always issues the same loads); its scales are
   // zeroed when the slot is consumed (not here: that would wait for the load right after requesting it),
   // which makes it contribute exactly 0
+  // Every offset is 32 bits wide (the launcher checks that the packed weights end below 4 GiB) and made of a part
+  // of the lane that never changes and a part of the wave (slice, column tile: scalar arithmetic): a request costs
+  // one vector addition.  (With 64-bit offsets the compiler keeps base + lane part in a register pair per operand and
+  // adds the wave's part to it with 64-bit vector additions: 110 instructions of address arithmetic per slot of four
+  // tiles against the 224 of its conversion.)
+  const uint32_t m2_lane[2] = {m_lane[0] * 2, m_lane[1] * 2};
+  // rows staged per slot: copy q fills LDS bytes [1024 q, 1024 q + 1024) of the slot, lane l the 16 bytes at 16 l;
+  // a last slice with two units only fetches its first pair twice
+  uint32_t a_copy[(AM == kRowsPerSlotInLds) ? 4 * MT : 1][2];
+  if (AM == kRowsPerSlotInLds) {
+#pragma unroll
+    for (int q = 0; q < 4 * MT; ++q) {
+      const int rr = 8 * q + (lane >> 3);  // (pair, row) index inside the slot
+      const int row = rr % kSlotRows;
+      const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+      const uint32_t in_pair = (static_cast<uint32_t>(min(row, M - 1)) * K + (chunk >> 2) * 32 + (chunk & 3) * 8) * 2;
+      a_copy[q][0] = in_pair + (rr / kSlotRows) * 128;
+      a_copy[q][1] = in_pair;
+    }
+  }
 #define BLKQ4_LOAD_SLOT(dst_, d_, cg_, slice_, keep_, W_, S_, Z_)                                                \
   {                                                                                            \
     const int sl_ = min((slice_), last_slice);                                                 \
     const bool alt_ = rem != 0 && sl_ == last_slice;                                           \
     const uint32_t wl_ = alt_ ? w_lane[1] : w_lane[0];                                         \
     const uint32_t ml_ = alt_ ? m_lane[1] : m_lane[0];                                         \
-    const size_t keep64_ = static_cast<size_t>(static_cast<long long>(keep_));                 \
+    const uint32_t ml2_ = alt_ ? m2_lane[1] : m2_lane[0];                                      \
+    const uint32_t keep32_ = static_cast<uint32_t>(keep_);                                     \
     if (AM == kRowsPerSlotInLds) {                                                             \
-      /* copy q: LDS bytes [1024 q, 1024 q + 1024) of the slot, lane l the 16 bytes at 16 l; */ \
-      /* requested before the slot's weights, so whoever has the weights has the rows        */ \
+      /* requested before the slot's weights, so whoever has the weights has the rows */       \
       _Pragma("unroll") for (int q = 0; q < 4 * MT; ++q) {                                     \
-        const int rr_ = 8 * q + (lane >> 3);             /* (pair, row) index inside the slot */ \
-        const int row_ = rr_ % kSlotRows;                                                      \
-        const int chunk_ = (lane & 7) ^ ((row_ >> 1) & 7);                                     \
-        const int u_ = 4 * sl_ + 2 * (rr_ / kSlotRows) + (chunk_ >> 2);                        \
-        const int ug_ = (u_ < units) ? u_ : (u_ & wrap_mask);                                  \
         async_copy_16(__builtin_amdgcn_readfirstlane(lds0 + (wave * DEPTH + (d_)) * kSlotBytes + q * 1024), A, \
-                      (static_cast<uint32_t>(min(row_, M - 1)) * K + ug_ * 32 + (chunk_ & 3) * 8) * 2); \
+                      (alt_ ? a_copy[q][1] : a_copy[q][0]) + static_cast<uint32_t>(sl_) * 256u); \
       }                                                                                        \
     }                                                                                          \
     _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                           \
@@ -293,23 +308,25 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       /* not stored                                                                                */ \
       const int tile_ = ((cg_) * kTileWaves + wt) * NT + t;                                    \
       const int tu_ = (tile_ < tiles) ? tile_ : (cg_) * (kTileWaves * NT);                     \
-      const size_t wu_ = ((static_cast<size_t>(4 * sl_) * N + tu_ * 16) * 16) & keep64_;       \
-      (dst_).w[t] = load_weights(W_, wu_ + wl_);                                               \
+      const uint32_t wu_ = ((static_cast<uint32_t>(4 * sl_) * N + tu_ * 16) * 16u) & keep32_;  \
+      (dst_).w[t] = load_weights(W_, static_cast<size_t>(wu_ + wl_));                          \
       if (ROW) {                                                                               \
-        const size_t mu_ = (static_cast<size_t>(tu_ * 16 / BS) * K + sl_ * 128) & keep64_;     \
+        const uint32_t mu_ = (static_cast<uint32_t>(tu_ * 16 / BS) * K + sl_ * 128) & keep32_; \
+        const uint32_t so_ = mu_ * 2 + ml2_;                                                   \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                        \
-          (dst_).rs[ROW ? t : 0][q] = load_16(S_, mu_ * 2 + ml_ * 2 + 16 * q);                 \
+          (dst_).rs[ROW ? t : 0][q] = load_16(S_, static_cast<size_t>(so_) + 16 * q);          \
         }                                                                                      \
         if (HAS_ZP) {                                                                          \
+          const uint32_t zo_ = mu_ + ml_;                                                      \
           _Pragma("unroll") for (int q = 0; q < 2; ++q) {                                      \
-            (dst_).rz[ROW ? t : 0][q] = load_16(Z_, mu_ + ml_ + 16 * q);                       \
+            (dst_).rz[ROW ? t : 0][q] = load_16(Z_, static_cast<size_t>(zo_) + 16 * q);        \
           }                                                                                    \
         }                                                                                      \
       } else {                                                                                 \
         _Pragma("unroll") for (int q = 0; q < kMeta; ++q) {                                    \
-          const size_t mu_ = (static_cast<size_t>(kBlocksPerSlice * sl_ + q) * N + tu_ * 16) & keep64_; \
-          (dst_).sc[t][ROW ? 0 : q] = load_u16(S_, mu_ * 2 + ml_ * 2);                         \
-          (dst_).zp[t][ROW ? 0 : q] = HAS_ZP ? load_u8(Z_, mu_ + ml_) : 8u;                    \
+          const uint32_t mu_ = (static_cast<uint32_t>(kBlocksPerSlice * sl_ + q) * N + tu_ * 16) & keep32_; \
+          (dst_).sc[t][ROW ? 0 : q] = load_u16(S_, static_cast<size_t>(mu_ * 2 + ml2_));       \
+          (dst_).zp[t][ROW ? 0 : q] = HAS_ZP ? load_u8(Z_, static_cast<size_t>(mu_ + ml_)) : 8u; \
         }                                                                                      \
       }                                                                                        \
     }                                                                                          \
@@ -638,6 +655,8 @@ int launch_kernel(const blkq4_gemm_args* a) {
   X(4, 1, 1, 4, BLKQ4_W, 1)                                                                                \
   /* wide layers, rows staged per slice */                                                                 \
   X(2, 4, 1, 4, BLKQ4_P, 4) X(2, 4, 1, 8, BLKQ4_P, 8)                                                      \
+  X(2, 5, 1, 4, BLKQ4_P, 4) X(2, 6, 1, 4, BLKQ4_P, 4) X(2, 7, 1, 4, BLKQ4_P, 4)                            \
+  X(2, 5, 1, 8, BLKQ4_P, 8) X(2, 6, 1, 8, BLKQ4_P, 8) X(2, 7, 1, 8, BLKQ4_P, 8)                            \
   /* up to 16 rows, the waves split K */                                                                   \
   X(4, 1, 1, 8, BLKQ4_W, 8) X(4, 2, 1, 8, BLKQ4_W, 8) X(4, 3, 1, 8, BLKQ4_W, 8) X(2, 1, 1, 8, BLKQ4_W, 8)  \
   X(2, 1, 1, 16, BLKQ4_W, 16) X(2, 2, 1, 16, BLKQ4_W, 16) X(2, 3, 1, 16, BLKQ4_W, 16)                      \
@@ -672,7 +691,8 @@ int launch_skinny(const blkq4_gemm_args* a) {
 
 extern "C" int BLKQ4_SKINNY_ENTRY(const blkq4_gemm_args* a) {
   if (a->m < 1 || a->m > kStreamingMaxRows || (a->n % 16) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
-  if (a->n > (1 << 26)) return static_cast<int>(hipErrorInvalidValue);  // a lane's offset inside a slice (up to 8 n rows of 16 bytes) is 32 bits wide
+  // every offset is 32 bits wide: the packed weights (K N / 2 bytes) end below 4 GiB
+  if (static_cast<uint64_t>(a->k) * static_cast<uint64_t>(a->n) > kStreamingMaxWeights) return static_cast<int>(hipErrorInvalidValue);
   if (!a->column_wise) {
     // blocks along N: a 16-column tile lies inside one block, and the meta data are fetched 16 bytes at a time
     if ((a->n % a->block_size) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 15u) != 0 ||

@@ -150,6 +150,8 @@ EXACT_CASES = [
     (64, True, 300, 4128, 192), (16, True, 500, 2080, 128), (32, False, 257, 4096, 64), (32, True, 1100, 4160, 128),
     (64, True, 48, 28672, 256), (32, False, 64, 36864, 128), (16, False, 32, 28672, 2624), (32, True, 24, 36864, 2624),
     (64, True, 768, 1056, 576), (16, True, 129, 1056, 576),
+    # five to seven column tiles per workgroup (wide layers, rows staged per slice)
+    (64, True, 16, 18432, 1088), (32, False, 9, 22016, 1088), (16, True, 12, 28672, 1216), (32, True, 16, 57344, 1024),
 ]
 
 

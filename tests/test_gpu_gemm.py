@@ -107,10 +107,25 @@ SIX_AND_EIGHT_TILE_CASES = [
     (32, True, 33, 11040, 2176), (64, False, 60, 14336, 4160),
 ]
 
+# five to sixteen rows on wide layers, rows staged per slice: five, six and seven column tiles per workgroup of four
+# or eight waves (as many as give every compute unit the same number of tiles), a last slice of two units only
+# (K = 64 mod 128), a last workgroup with tiles missing
+FIVE_TO_SEVEN_TILE_CASES = [
+    (64, True, 16, 18432, 4096), (32, False, 9, 22016, 2048), (16, True, 16, 28672, 1088), (32, True, 13, 36864, 4160),
+    (64, True, 16, 57344, 2048), (32, True, 6, 22016, 8192), (64, False, 5, 20480, 8256), (64, True, 11, 40960, 1088),
+    (32, True, 16, 24608, 4096),
+]
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + SMALL_TILE_CASES + WIDE_TILE32_CASES + LONG_K_CASES + VERY_WIDE_CASES + SIX_AND_EIGHT_TILE_CASES)
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + SMALL_TILE_CASES + WIDE_TILE32_CASES + LONG_K_CASES + VERY_WIDE_CASES + SIX_AND_EIGHT_TILE_CASES + FIVE_TO_SEVEN_TILE_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", FIVE_TO_SEVEN_TILE_CASES)
+def test_five_to_seven_tile_cases_run_the_shapes_they_are_meant_for(capi, bs, has_offsets, m, n, k):
+    text = capi.gemm_plan(bs, True, m, n, k, has_offsets)[2]
+    assert text.startswith("streaming:") and any(f"{t} column tile(s) x 16 rows" in text for t in (5, 6, 7)) and "rows staged per slice" in text
 
 
 def gaussian_problem(seed, m, n, k):
