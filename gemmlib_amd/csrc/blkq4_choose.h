@@ -467,11 +467,32 @@ inline double tile_estimate_us(const TileShape& t, int k) {
   return us;
 }
 
+// Tiles of one row tile (up to 64 rows, blocks along K): a workgroup walks through K at a pace set by latency, not
+// by the chip's load.  Measured over N = 2048 ... 32768 (16 -> 256 workgroups of 128 columns, four waves and four
+// producer waves): K = 1024 (16 k tiles) 7.2 -> 8.1 us with up to 32 rows, 6.8 -> 9.2 with up to 64; K = 2048 11.5
+// -> 13.1 and 10.7 -> 15.3; K = 4096 20.0 -> 23.1 and 18.4 -> 26.7; 256 columns with eight waves 31.9 -> 34.5 us at
+// K = 4096.  Whole rounds of 256 workgroups.
+inline double one_row_tile_estimate_us(const TileShape& t, int k) {
+  const long busy = t.tiles < kComputeUnits ? t.tiles : kComputeUnits;
+  double step, fixed;
+  if (t.wn != 4) {
+    step = 0.50 + 0.00015 * busy;
+    fixed = 1.0;
+  } else if (t.rt == 1) {
+    step = 0.27 + 0.00017 * busy;
+    fixed = 2.6 + 0.002 * busy;
+  } else {
+    step = 0.325 + 0.00015 * busy;
+    fixed = 1.3 + 0.008 * busy;
+  }
+  return static_cast<double>(ceil_div(t.tiles, kComputeUnits)) * (fixed + (k / 64) * step);
+}
+
 // The tile kernel's plan: the shape with the smallest estimate; when its last round of tiles would leave most
 // of the chip idle and the estimate says it pays, those last `split_tiles` tiles are each shared out over
 // split_k workgroups.  Up to 64 rows with blocks along K: tiles of one row tile, which fetch every packed
-// weight once (128 columns with four waves and four producer waves when such tiles fill the chip in one
-// round, else 256 columns with eight waves; M = 64, K = 4096, N = 28672: 34.7 against 26.3 us).
+// weight once (128 columns with four waves and four producer waves, or 256 columns with eight waves, whichever
+// one_row_tile_estimate_us() expects to be faster: the narrow ones up to one round of them, N = 32768).
 inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspace_capacity) {
   TileShape best{};
   auto shape = [&](int rt, int nt, int wm, int wn, int pw) {
@@ -482,9 +503,9 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
     return t;
   };
   if (column_wise && m <= 64) {
-    const bool one_round_of_128 = n / 128 >= 224 && n / 128 <= kComputeUnits;
     const int rt = m <= 32 ? 1 : 2;
-    return one_round_of_128 ? shape(rt, 1, 1, 4, 4) : shape(rt, 1, 1, 8, 0);
+    const TileShape narrow = shape(rt, 1, 1, 4, 4), wide = shape(rt, 1, 1, 8, 0);
+    return one_row_tile_estimate_us(narrow, k) <= one_row_tile_estimate_us(wide, k) ? narrow : wide;
   }
   const int kt = k / 64;
   double best_us = 0.0, best_unsplit_us = 0.0;
@@ -529,23 +550,26 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
   // its offsets into the packed weights (K N / 2 bytes) are 32 bits wide
   if (static_cast<uint64_t>(k) * static_cast<uint64_t>(n) > kStreamingMaxWeights) return false;
   if (m <= 16) return true;
-  if (m <= 32) {
-    // 17 to 32 rows: the streaming kernel wins unless it cannot keep the rows in LDS for all of K (it then
-    // fetches them again for every column group) and the problem is wide enough for the tile kernel's 32-row
-    // tiles to fill the chip: M = 32, K = 4096, N = 28672 takes 27.3 us streaming and 23.1 us in tiles, with
-    // N = 65536 53.7 and 39.5 us.
-    const bool rows_fit = 32L * k * 2 <= static_cast<long>(kMaxLdsBytes);
-    return !column_wise || rows_fit || n / 128 < 224;
-  }
   if (m > kStreamingMaxRows) return false;
   const long row_groups = s.row_groups;
-  // blocks along N: the streaming kernel converts with 23 instead of 13 instructions per 8 weights
+  const long streaming_groups = row_groups * ceil_div(n / 16, s.nt);
+  const long rounds = ceil_div(streaming_groups, kComputeUnits);
+  if (column_wise && m <= 64) {
+    // One or two row groups of 32, blocks along K: rounds of 256 workgroups, a workgroup's time growing with its column tiles
+    // and K.  Least squares over 142 measurements (M = 24 ... 64, K = 1024 ... 4096, N = 2048 ... 32768; within 15 %
+    // of all but a few, and of M = 128, K = N = 4096 and M = 40 ... 64, K = 8192, N = 16384 ... 18432, which were not
+    // among them); against the tile kernel's estimate it picks the faster kernel on all of them but for 0.04 % of
+    // the time.  (M = 64, N = 18432: K = 4096 29.8 us streaming, 23.8 in tiles; K = 1024 17.2 and 8.7.)
+    const double streaming_us = 3.2 + static_cast<double>(rounds) * (0.44 + s.nt * (0.69 + 0.37 * (static_cast<double>(k) / 1024.0)));
+    return streaming_us < tile_us;
+  }
+  if (m <= 32) return true;
+  // more row groups, and blocks along N, where the streaming kernel converts with 23 instead of 13 instructions per 8
+  // weights
   double streaming_us = (column_wise ? 2.8 : 5.6) * static_cast<double>(row_groups) * (static_cast<double>(n) / 4096.0) *
                         (static_cast<double>(k) / 4096.0);
-  const long streaming_groups = row_groups * ceil_div(n / 16, s.nt);
   if (streaming_groups > kComputeUnits) {
-    streaming_us *= static_cast<double>(ceil_div(streaming_groups, kComputeUnits)) /
-                    (static_cast<double>(streaming_groups) / kComputeUnits);
+    streaming_us *= static_cast<double>(rounds) / (static_cast<double>(streaming_groups) / kComputeUnits);
   }
   return streaming_us < tile_us;
 }
@@ -562,7 +586,8 @@ inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t wo
   }
   if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k);
   c.t = tile_plan(column_wise, m, n, k, workspace_capacity);
-  c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_estimate_us(c.t, k)) ? kFamilyStreaming : kFamilyTile;
+  const double tile_us = (column_wise && m <= 64) ? one_row_tile_estimate_us(c.t, k) : tile_estimate_us(c.t, k);
+  c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_us) ? kFamilyStreaming : kFamilyTile;
   return c;
 }
 

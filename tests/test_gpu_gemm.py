@@ -68,10 +68,13 @@ LARGE_TILE_CASES = [(64, True, 4096, 4096, 128), (16, True, 4000, 4128, 64), (32
 SMALL_TILE_CASES = [(64, True, 300, 4128, 192), (16, True, 500, 2080, 128), (32, False, 257, 4096, 64)]
 # very wide N and rows that the streaming kernel cannot keep in LDS for all of K: up to 16 rows it takes more
 # column tiles per workgroup (the rows are fetched once per workgroup and slice), 17 to 64 rows go to the tile
-# kernel's 32- and 64-row tiles (128 columns when those fill the chip in one round, else 256)
+# kernel's 32- and 64-row tiles (128 columns up to one round of them, else 256)
 WIDE_TILE32_CASES = [
     (64, True, 16, 28672, 5184), (32, True, 9, 28704, 5248), (16, False, 32, 28672, 2624), (64, False, 20, 28672, 2688),
     (32, True, 24, 36864, 2624), (64, True, 48, 28672, 256), (32, False, 64, 36864, 128),
+    # the 128-column tiles of one row tile half-filling the chip (144 and 160 workgroups), where two rounds of streaming
+    # workgroups would take longer
+    (64, True, 64, 18432, 1024), (32, False, 24, 28672, 1088), (16, True, 48, 20480, 2048), (64, False, 33, 18464, 4096),
 ]
 WIDE_SKINNY_CASES = [
     (16, True, 12, 4128, 128), (32, True, 8, 8224, 128), (64, False, 3, 8224, 192), (32, False, 5, 28672, 64),
