@@ -87,23 +87,23 @@ DESCRIPTION = {
 # figure of a workload is reported only while the library still picks the kernel it was taken from (TRAFFIC_KERNEL).
 COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65552.0, "WRITE_SIZE": 1.0}
 COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
-    "C4": (44108.2, 16384.6),
-    "C2": (4428.1, 8.0),
+    "C4": (44108.3, 16384.5),
+    "C2": (4429.6, 8.0),
     "C3": (13653.6, 344.0),
-    "C5": (860404.6, 229384.7),
-    "C5_prepack": (229443.8, 157731.3),
-    "C4r": (44108.6, 16387.8),
-    "C2r": (4431.1, 8.0),
-    "C1": (875.0, 128.0),
-    "M128": (8661.1, 1024.0),
-    "M256": (24123.1, 11274.2),
-    "M512": (37925.5, 4542.0),
-    "M768N11K": (60847.5, 16512.7),
-    "M256K11K": (43356.1, 19401.4),
-    "V128K": (136348.9, 252.3),
-    "B16": (63817.2, 896.0),
+    "C5": (860383.9, 229387.1),
+    "C5_prepack": (229443.7, 157730.3),
+    "C4r": (44108.6, 16387.5),
+    "C2r": (4428.1, 8.0),
+    "C1": (869.5, 128.0),
+    "M128": (8650.6, 1024.0),
+    "M256": (24123.1, 11273.8),
+    "M512": (37925.5, 4538.0),
+    "M768N11K": (60847.5, 16512.5),
+    "M256K11K": (43356.1, 19392.0),
+    "V128K": (136348.9, 251.0),
+    "B16": (64098.7, 896.0),
     "C4b": (44128.5, 16386.3),
-    "C2b": (4440.1, 8.0),
+    "C2b": (4441.1, 8.0),
 }
 
 
@@ -117,7 +117,7 @@ TRAFFIC_KERNEL = {  # what blkq4_gemm_plan_sm80 said the workload runs when its 
     "C2r": "decode (blocks along N): 4 waves splitting K, 8 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
     "M128": "streaming: 8 waves splitting K, 4 column tile(s) x 32 rows, 2 slices in flight, rows staged per slice, 4 row group(s), 256 workgroups",
     "V128K": "decode: 8 waves splitting K, 4 slices requested by each, 2 column tile(s) x 1 row(s), 4008 workgroups",
-    "B16": "streaming: 4 waves splitting K, 4 column tile(s) x 16 rows, 2 slices in flight, rows staged per slice, 1 row group(s), 448 workgroups",
+    "B16": "streaming: 8 waves splitting K, 7 column tile(s) x 16 rows, 2 slices in flight, rows staged per slice, 1 row group(s), 256 workgroups",
     "C4b": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
     "C2b": "decode: 4 waves splitting K, 8 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
     "M256": "tile: 64 x 128, 4 + 4 waves, 128 tiles, the last 128 in 2 parts (workspace 8404992 bytes)",
