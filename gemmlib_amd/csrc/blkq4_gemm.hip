@@ -46,6 +46,8 @@
 
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "blkq4_choose.h"
 #include "blkq4_dequant.h"
 #include "blkq4_device.h"
@@ -515,14 +517,17 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   constexpr int kCut2 = (kCopySteps == 4) ? kOps * 2 / 4 : (kCopySteps == 2) ? kOps : 0;
   constexpr int kCut3 = kOps * 3 / 4;
 
-  for (int kt = 0; kt < KT; ++kt) {
-    const int stage = kt % kStages;
-    const uint32_t sa = stage * St::kBytes;                               // tile kt: offset of its ring slot
-    const uint32_t sn = ((kt + 1) % kStages) * St::kBytes;                // tile kt + 1
+  // One k tile, in ring slot `stage` (a compile-time constant: the loop below is unrolled by the ring's depth by
+  // hand -- the compiler does not unroll a loop with barriers whose trip count it does not know -- so that the
+  // slots' offsets are constants and the hand-over of the next tile's words and constants costs no copies).
+  auto k_tile = [&](const int kt, auto stage_tag) __attribute__((always_inline)) {
+    constexpr int stage = decltype(stage_tag)::value;
+    constexpr uint32_t sa = stage * St::kBytes;                           // tile kt: offset of its ring slot
+    constexpr uint32_t sn = ((stage + 1) % kStages) * St::kBytes;         // tile kt + 1
     const int copy_tile = min(kt + kDistance, KT - 1);                    // clamped: re-fetches the last tile
-    const int copy_stage = (kt + kDistance) % kStages;
+    constexpr int copy_stage = (stage + kDistance) % kStages;
     const int late_tile = min(kt + kDistance - 1, KT - 1);                // the group begun in the previous tile
-    const int late_stage = (kt + kDistance - 1) % kStages;
+    constexpr int late_stage = (stage + kDistance - 1) % kStages;
     BLKQ4_PIN();
 
     // step 0: uses buffers 0; prepares step 1
@@ -551,6 +556,14 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
         if constexpr (kBF) bdc[t][q] = bndc[t][q];
         else dc[t][q] = ndc[t][q];
       }
+    }
+  };
+  for (int kt0 = 0; kt0 < KT; kt0 += kStages) {
+    k_tile(kt0, std::integral_constant<int, 0>{});
+    if (kt0 + 1 < KT) k_tile(kt0 + 1, std::integral_constant<int, 1>{});
+    if (kt0 + 2 < KT) k_tile(kt0 + 2, std::integral_constant<int, 2>{});
+    if constexpr (kStages == 4) {
+      if (kt0 + 3 < KT) k_tile(kt0 + 3, std::integral_constant<int, 3>{});
     }
   }
   if (PW == 0) wait_vmcnt<0>();  // the clamped re-fetches of the last tile are still in flight
