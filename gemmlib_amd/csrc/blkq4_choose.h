@@ -469,21 +469,21 @@ inline double tile_estimate_us(const TileShape& t, int k) {
 
 // Tiles of one row tile (up to 64 rows, blocks along K): a workgroup walks through K at a pace set by latency, not
 // by the chip's load.  Measured over N = 2048 ... 32768 (16 -> 256 workgroups of 128 columns, four waves and four
-// producer waves): K = 1024 (16 k tiles) 7.2 -> 8.1 us with up to 32 rows, 6.8 -> 9.2 with up to 64; K = 2048 11.5
-// -> 13.1 and 10.7 -> 15.3; K = 4096 20.0 -> 23.1 and 18.4 -> 26.7; 256 columns with eight waves 31.9 -> 34.5 us at
+// producer waves): K = 1024 (16 k tiles) 6.5 -> 7.3 us with up to 32 rows, 7.3 -> 9.5 with up to 64; K = 2048 10.0 ->
+// 12.1 and 11.0 -> 15.8; K = 4096 17.5 -> 20.5 and 19.4 -> 27.4; 256 columns with eight waves 28.6 -> 31.7 us at
 // K = 4096.  Whole rounds of 256 workgroups.
 inline double one_row_tile_estimate_us(const TileShape& t, int k) {
   const long busy = t.tiles < kComputeUnits ? t.tiles : kComputeUnits;
   double step, fixed;
   if (t.wn != 4) {
-    step = 0.50 + 0.00015 * busy;
-    fixed = 1.0;
+    step = 0.40 + 0.0003 * busy;
+    fixed = 2.9;
   } else if (t.rt == 1) {
-    step = 0.27 + 0.00017 * busy;
-    fixed = 2.6 + 0.002 * busy;
+    step = 0.22 + 0.0002 * busy;
+    fixed = 2.85;
   } else {
-    step = 0.325 + 0.00015 * busy;
-    fixed = 1.3 + 0.008 * busy;
+    step = 0.25 + (busy > 128 ? (busy - 128) * 0.00097 : 0.0);
+    fixed = 3.3;
   }
   return static_cast<double>(ceil_div(t.tiles, kComputeUnits)) * (fixed + (k / 64) * step);
 }
@@ -555,11 +555,12 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
   const long streaming_groups = row_groups * ceil_div(n / 16, s.nt);
   const long rounds = ceil_div(streaming_groups, kComputeUnits);
   if (column_wise && m <= 64) {
-    // One or two row groups of 32, blocks along K: rounds of 256 workgroups, a workgroup's time growing with its column tiles
-    // and K.  Least squares over 142 measurements (M = 24 ... 64, K = 1024 ... 4096, N = 2048 ... 32768; within 15 %
-    // of all but a few, and of M = 128, K = N = 4096 and M = 40 ... 64, K = 8192, N = 16384 ... 18432, which were not
-    // among them); against the tile kernel's estimate it picks the faster kernel on all of them but for 0.04 % of
-    // the time.  (M = 64, N = 18432: K = 4096 29.8 us streaming, 23.8 in tiles; K = 1024 17.2 and 8.7.)
+    // One or two row groups of 32, blocks along K: rounds of 256 workgroups, a workgroup's time growing with its
+    // column tiles and K.  Least squares over 142 measurements (M = 24 ... 64, K = 1024 ... 4096, N = 2048 ... 32768;
+    // within 15 % of all but a few, and of M = 128, K = N = 4096 and M = 40 ... 64, K = 8192, N = 16384 ... 18432, which
+    // were not among them); against the tile kernel's estimate it picks the slower kernel for 0.2 % of the time
+    // on them.  (M = 64, N = 18432: K = 4096 29.8 us streaming, 19.6 in tiles; K = 1024 17.2 and 8.7.  With the same
+    // formula for three and four row groups M = 96, N = 8192 went to the tile kernel and took 20.1 instead of 19.4 us.)
     const double streaming_us = 3.2 + static_cast<double>(rounds) * (0.44 + s.nt * (0.69 + 0.37 * (static_cast<double>(k) / 1024.0)));
     return streaming_us < tile_us;
   }

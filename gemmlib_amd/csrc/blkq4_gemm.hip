@@ -114,10 +114,14 @@ struct Stage {
   static constexpr int kMTotal = ROW ? kRowScaleOps + kRowZpOps : WN * kBlocks;
   static constexpr int kMOps = (kMTotal + kCopiers - 1) / kCopiers;
   static constexpr int kOps = kAOps + kBOps + kMOps;
-  // ring of k tiles in LDS, requested kDistance tiles ahead of the one being consumed (deeper rings were
-  // measured and lose: up to eight slots, M = 256, K = N = 4096: 64 x 128 tiles 18.7 -> 20.4 us, 128 x 128 tiles
-  // 24.3 -> 28.3 us; C4 unchanged)
-  static constexpr int kStages = (4 * kBytes <= 160 * 1024) ? 4 : 3;
+  // Ring of k tiles in LDS, requested kDistance tiles ahead of the one being consumed.  A tile must have landed one
+  // k tile before it is consumed (the barrier in the middle of the tile before publishes it), so with four slots a
+  // request has two k tiles' time to complete: enough for the large tiles, whose k tile takes 0.6 us and more, not
+  // for the small ones (0.3 us).  Eight slots for those: M = 300, K = N = 4096 21.2 -> 18.8 us, M = 64, N = 18432 23.3 ->
+  // 19.6, M = 256 19.0 -> 18.3, M = 512 (256 workgroups: bound by what L2 delivers) 23.6 -> 23.2.  Six slots for the
+  // 128 x 128 tiles change nothing (+- 2 %), eight for the 256-column tiles of one row tile lose 5 %.
+  static constexpr bool kDeep = PW > 0 && RT * NT <= 2;
+  static constexpr int kStages = (kDeep && 8 * kBytes <= 160 * 1024) ? 8 : (4 * kBytes <= 160 * 1024) ? 4 : 3;
   static constexpr int kDistance = kStages - 1;  // the slot being refilled is the one nobody reads
   static_assert((kDistance - 1) * kOps <= 63, "more copies in flight than the counter holds");
 };
@@ -562,9 +566,18 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
     k_tile(kt0, std::integral_constant<int, 0>{});
     if (kt0 + 1 < KT) k_tile(kt0 + 1, std::integral_constant<int, 1>{});
     if (kt0 + 2 < KT) k_tile(kt0 + 2, std::integral_constant<int, 2>{});
-    if constexpr (kStages == 4) {
+    if constexpr (kStages > 3) {
       if (kt0 + 3 < KT) k_tile(kt0 + 3, std::integral_constant<int, 3>{});
     }
+    if constexpr (kStages > 4) {
+      if (kt0 + 4 < KT) k_tile(kt0 + 4, std::integral_constant<int, 4>{});
+      if (kt0 + 5 < KT) k_tile(kt0 + 5, std::integral_constant<int, 5>{});
+    }
+    if constexpr (kStages > 6) {
+      if (kt0 + 6 < KT) k_tile(kt0 + 6, std::integral_constant<int, 6>{});
+      if (kt0 + 7 < KT) k_tile(kt0 + 7, std::integral_constant<int, 7>{});
+    }
+    static_assert(kStages == 3 || kStages == 4 || kStages == 6 || kStages == 8, "unrolled by hand for these ring depths");
   }
   if (PW == 0) wait_vmcnt<0>();  // the clamped re-fetches of the last tile are still in flight
 #undef BLKQ4_COPY_OP
