@@ -87,22 +87,22 @@ DESCRIPTION = {
 # figure of a workload is reported only while the library still picks the kernel it was taken from (TRAFFIC_KERNEL).
 COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65552.0, "WRITE_SIZE": 1.0}
 COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
-    "C4": (44108.3, 16384.5),
+    "C4": (44138.2, 16386.4),
     "C2": (4429.6, 8.0),
     "C3": (13653.6, 344.0),
-    "C5": (860383.9, 229387.1),
+    "C5": (860409.6, 229384.7),
     "C5_prepack": (229443.7, 157730.3),
-    "C4r": (44108.6, 16387.5),
+    "C4r": (44141.6, 16386.0),
     "C2r": (4428.1, 8.0),
     "C1": (869.5, 128.0),
     "M128": (8650.6, 1024.0),
-    "M256": (24123.1, 11273.8),
-    "M512": (37925.5, 4538.0),
-    "M768N11K": (60847.5, 16512.5),
-    "M256K11K": (43356.1, 19392.0),
+    "M256": (24163.1, 11216.5),
+    "M512": (37966.5, 4266.3),
+    "M768N11K": (60858.5, 16514.9),
+    "M256K11K": (43371.1, 19433.4),
     "V128K": (136348.9, 251.0),
     "B16": (64098.7, 896.0),
-    "C4b": (44128.5, 16386.3),
+    "C4b": (44167.5, 16387.6),
     "C2b": (4441.1, 8.0),
 }
 
