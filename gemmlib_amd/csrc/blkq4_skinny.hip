@@ -468,31 +468,24 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
       // all fragment reads are requested before the conversion starts (left to itself the compiler puts each read
       // right before the MFMA that needs it, which then waits out the whole LDS latency)
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const uint32_t words[4] = {cur.w[t].x, cur.w[t].y, cur.w[t].z, cur.w[t].w};
+      // the constants of the tile being converted (blocks along K)
+      DequantConsts dc[kMeta];
+      Bf16Consts bc[kMeta];
+      // word j of tile t as the eight values of the MFMA's weight operand (for bf16: their bits)
+      auto convert = [&](const int t, const int j) -> half8_t {
+        const uint32_t word = vec_word(cur.w[t], j);
         if constexpr (kBF && !ROW) {
-          Bf16Consts bc[kMeta];
+          if (j == 0) {
 #pragma unroll
-          for (int q = 0; q < kMeta; ++q) bc[q] = make_bf16_consts(cur.sc[t][q] & okm, cur.zp[t][q]);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const bf16x8_t wf = dequant_word_bf16(words[j], bc[(kMeta == 2) ? (j >> 1) : 0], masks);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-              acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, as_bf16x8(af[mt][j]), acc[t][mt], 0, 0, 0);
-            }
+            for (int q = 0; q < kMeta; ++q) bc[q] = make_bf16_consts(cur.sc[t][q] & okm, cur.zp[t][q]);
           }
-          continue;
-        }
-        DequantConsts dc[kMeta];
-        if (!ROW) {
+          return __builtin_bit_cast(half8_t, dequant_word_bf16(word, bc[(kMeta == 2) ? (j >> 1) : 0], masks));
+        } else {
+          if (!ROW && j == 0) {
 #pragma unroll
-          for (int q = 0; q < kMeta; ++q) dc[q] = make_dequant_consts(cur.sc[t][ROW ? 0 : q] & okm, cur.zp[t][ROW ? 0 : q]);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint32_t y = words[j] >> 8;
+            for (int q = 0; q < kMeta; ++q) dc[q] = make_dequant_consts(cur.sc[t][ROW ? 0 : q] & okm, cur.zp[t][ROW ? 0 : q]);
+          }
+          const uint32_t y = word >> 8;
           half2_t p[4];
           if (ROW) {
             // word j is rows 8 hh .. 8 hh + 7 of 16-row group j / 2 of the unit: pair i has its scales in
@@ -506,7 +499,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const uint32_t zpair = HAS_ZP ? ((zw[i] >> (8 * hh)) & 0x00ff00ffu) : 0x00080008u;
-              const uint32_t src = (i >= 2) ? y : words[j];
+              const uint32_t src = (i >= 2) ? y : word;
               const half2_t s2 = as_half2(sw[2 * i + hh] & okm);
               // q - zp of the pair, exact
               const half2_t d = ((i & 1) == 0)
@@ -520,24 +513,37 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
             }
           } else {
             const DequantConsts& c = dc[(kMeta == 2) ? (j >> 1) : 0];
-            p[0] = dequant_pair(words[j], 0, c, masks);
-            p[1] = dequant_pair(words[j], 1, c, masks);
+            p[0] = dequant_pair(word, 0, c, masks);
+            p[1] = dequant_pair(word, 1, c, masks);
             p[2] = dequant_pair(y, 2, c, masks);
             p[3] = dequant_pair(y, 3, c, masks);
           }
           half8_t wf;
           wf[0] = p[0][0]; wf[1] = p[0][1]; wf[2] = p[1][0]; wf[3] = p[1][1];
           wf[4] = p[2][0]; wf[5] = p[2][1]; wf[6] = p[3][0]; wf[7] = p[3][1];
+          return wf;
+        }
+      };
+      // The next word is converted before this one's MFMAs are issued: a conversion's last instruction would otherwise
+      // feed the MFMA right behind it, and the wait states that costs were an s_nop per word (21 of a slot's 355
+      // instructions with four tiles).
+      half8_t wf = convert(0, 0);
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            if constexpr (kBF) {
-              acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf), as_bf16x8(af[mt][j]),
-                                                                  acc[t][mt], 0, 0, 0);
-            } else {
-              acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, as_half8(af[mt][j]), acc[t][mt], 0, 0, 0);
-            }
+      for (int x = 0; x < 4 * NT; ++x) {
+        const int t = x >> 2, j = x & 3;
+        half8_t next = wf;
+        if (x + 1 < 4 * NT) next = convert((x + 1) >> 2, (x + 1) & 3);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          if constexpr (kBF) {
+            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf), as_bf16x8(af[mt][j]),
+                                                                acc[t][mt], 0, 0, 0);
+          } else {
+            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, as_half8(af[mt][j]), acc[t][mt], 0, 0, 0);
           }
         }
+        wf = next;
       }
   };
 
