@@ -175,10 +175,8 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   const int wt = (kSplit == 1) ? wave : 0;  // and its column tiles the wt-th NT of the column group
   const int my_slices = (slices - ws + kSplit - 1) / kSplit;
 
-  const int wrap_mask = (1 << (31 - __builtin_clz(units))) - 1;  // any index & wrap_mask is < units
-
-  // Addresses are a wave-uniform 64-bit part (slice and column tile: scalar arithmetic) plus a 32-bit part
-  // of the lane that never changes: (k-unit of the slice g, column nl).  Only in the last slice, when it has
+  // Addresses are a wave-uniform part (slice and column tile: scalar arithmetic) plus a part of the lane that
+  // never changes, 32 bits each: (k-unit of the slice g, column nl).  Only in the last slice, when it has
   // rem < 4 units, the lanes past the end ask for unit g % rem instead (their scales are zeroed when the slot
   // is consumed), and a slot past the wave's last slice asks for the last slice once more.
   constexpr int kBlocksPerSlice = (BS == 64) ? 2 : (BS == 32) ? 4 : 8;
