@@ -97,6 +97,16 @@ inline uint32_t decode_grid(int n, int nt) {
   return static_cast<uint32_t>((groups + 63) / 64 * 64);
 }
 
+// Two to four rows with K >= 8192 on layers of 1376 to 3584 column tiles: the streaming kernel's workgroups of five to
+// seven tiles, all resident at once, beat the decode kernel's rounds of single tiles (same process, decode against
+// streaming: M = 4, K = 8192: N = 28672 27.6 -> 26.7 us, N = 57344 58.2 -> 52.2, blocks of 16 with zero-points,
+// N = 24576 31.0 -> 25.9; K = 11008, N = 28672 41.8 -> 34.0; M = 2, K = 16384, N = 28672 53.4 -> 44.7; the worst case
+// found, M = 3, N = 22016 without zero-points, 19.7 -> 20.5).  With one row, at K = 4096 and on wider layers the decode
+// kernel wins.
+inline bool streaming_takes_few_rows(int m, int n, int k) {
+  return m >= 2 && m <= 4 && k >= 8192 && n / 16 >= 1376 && n / 16 <= 3584;
+}
+
 // The decode kernel's shape for m rows, or false when it has none or the streaming kernel is expected to be
 // faster: blocks along K, at most kDecodeMaxRows rows, K in whole 128-deep slices, few enough of them for the waves
 // to request them all at once and for the rows to fit in LDS, and packed weights that 32-bit offsets reach.
@@ -142,6 +152,7 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
   }
   const int slices = k / 128;
   const int tiles = n / 16;
+  if (streaming_takes_few_rows(m, n, k)) return false;
   const int rows = m == 1 ? 1 : m <= 4 ? 4 : m <= 8 ? 8 : 16;
   int waves = 8;
   if (rows <= 4) {
@@ -326,7 +337,7 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
       return done();
     }
   }
-  if (!row && (!rows_fit || m > 4) && k >= 1024) {
+  if (!row && (!rows_fit || m > 4 || streaming_takes_few_rows(m, n, k)) && k >= 1024) {
     // Wide N and more than four rows, or K too long for the rows to stay in LDS: the rows are staged per
     // slice, a workgroup takes four column tiles (the rows are fetched again for every column group) and a
     // wave keeps two slices in flight, so that the slots are small enough for several workgroups per compute

@@ -117,6 +117,8 @@ FIVE_TO_SEVEN_TILE_CASES = [
     (64, True, 16, 18432, 4096), (32, False, 9, 22016, 2048), (16, True, 16, 28672, 1088), (32, True, 13, 36864, 4160),
     (64, True, 16, 57344, 2048), (32, True, 6, 22016, 8192), (64, False, 5, 20480, 8256), (64, True, 11, 40960, 1088),
     (32, True, 16, 24608, 4096),
+    # two to four rows with K >= 8192 take the same shapes
+    (64, True, 4, 22016, 8192), (32, False, 2, 28672, 8256), (16, True, 3, 24576, 8192),
 ]
 
 
