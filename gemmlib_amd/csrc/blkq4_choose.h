@@ -97,14 +97,20 @@ inline uint32_t decode_grid(int n, int nt) {
   return static_cast<uint32_t>((groups + 63) / 64 * 64);
 }
 
-// Two to four rows with K >= 8192 on layers of 1376 to 3584 column tiles: the streaming kernel's workgroups of five to
-// seven tiles, all resident at once, beat the decode kernel's rounds of single tiles (same process, decode against
-// streaming: M = 4, K = 8192: N = 28672 27.6 -> 26.7 us, N = 57344 58.2 -> 52.2, blocks of 16 with zero-points,
-// N = 24576 31.0 -> 25.9; K = 11008, N = 28672 41.8 -> 34.0; M = 2, K = 16384, N = 28672 53.4 -> 44.7; the worst case
-// found, M = 3, N = 22016 without zero-points, 19.7 -> 20.5).  With one row, at K = 4096 and on wider layers the decode
-// kernel wins.
+// Up to four rows on wide layers with long K: the streaming kernel's workgroups of four to seven tiles, all resident at
+// once, beat the decode kernel's rounds of single tiles
+//   - two to four rows, K >= 8192, 1376 to 3584 column tiles (same process, decode against streaming: M = 4, K = 8192:
+//     N = 28672 27.6 -> 26.7 us, N = 57344 58.2 -> 52.2, blocks of 16 with zero-points, N = 24576 31.0 -> 25.9; the worst
+//     case found, M = 3, N = 22016 without zero-points, 19.7 -> 20.5; one row: 23.1 against 24.3, stays);
+//   - one to four rows, K > 8192 (where the decode kernel needs sixteen waves), 832 to 1792 column tiles (M = 1:
+//     K = 16384, N = 28672 51.1 -> 45.5 us, N = 13312 29.7 -> 25.1; K = N = 28672 87.0 -> 75.8; K = 8256, N = 13312 18.4 ->
+//     14.9; K = 11008, N = 28672 with zero-points 42.6 -> 37.7, N = 14336 without 19.0 -> 20.6, the one loss found; on
+//     wider layers the decode kernel is ahead again: K = 11008, N = 36864 41.4 against 44.0).
+// At K = 4096 and on wider layers the decode kernel wins.
 inline bool streaming_takes_few_rows(int m, int n, int k) {
-  return m >= 2 && m <= 4 && k >= 8192 && n / 16 >= 1376 && n / 16 <= 3584;
+  const int tiles = n / 16;
+  if (m > 4) return false;
+  return (m >= 2 && k >= 8192 && tiles >= 1376 && tiles <= 3584) || (k > 8192 && tiles >= 832 && tiles <= 1792);
 }
 
 // The decode kernel's shape for m rows, or false when it has none or the streaming kernel is expected to be
