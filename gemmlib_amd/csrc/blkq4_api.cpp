@@ -16,6 +16,15 @@
 
 namespace {
 
+// Every kernel addresses the activations and the packed weights with 32-bit byte offsets.
+inline bool too_large(int m, int n, int k) {
+  return static_cast<uint64_t>(m) * static_cast<uint64_t>(k) * 2 >= (uint64_t{1} << 32) ||
+         static_cast<uint64_t>(k) * static_cast<uint64_t>(n) / 2 >= (uint64_t{1} << 32);
+}
+constexpr const char* kTooLarge =
+    "Kernel execution failed: Error Invalid Problem (activations of m * k * 2 bytes and packed weights of k * n / 2 bytes "
+    "must stay below 4 GiB)";
+
 inline void set_error(std::string* err, std::string&& text) {
   if (err) *err = std::move(text);
 }
@@ -273,6 +282,10 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
     set_error(err, "Null tensor pointer");
     return -1;
   }
+  if (too_large(m, n, k)) {
+    set_error(err, kTooLarge);
+    return -1;
+  }
 
   blkq4_gemm_args args{};
   args.block_size = block_size;
@@ -420,6 +433,10 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
   }
   if ((k % 64) != 0 || (k % krow) != 0 || (n % kcol) != 0 || (n % 32) != 0) {
     set_error(err, "Kernel execution failed: Error Invalid Problem");
+    return -1;
+  }
+  if (too_large(m, n, k)) {
+    set_error(err, kTooLarge);
     return -1;
   }
   const blkq4::Choice choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, blkq4_dev_workspace_capacity());

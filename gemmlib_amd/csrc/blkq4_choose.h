@@ -564,8 +564,9 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
 constexpr uint64_t kStreamingMaxWeights = uint64_t{1} << 33;
 
 inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const StreamingShape& s, double tile_us) {
-  // its offsets into the packed weights (K N / 2 bytes) are 32 bits wide
-  if (static_cast<uint64_t>(k) * static_cast<uint64_t>(n) > kStreamingMaxWeights) return false;
+  // its offsets into the packed weights (K N / 2 bytes) are 32 bits wide (so are the other kernels': the entry points
+  // refuse such problems before any kernel is chosen)
+  if (static_cast<uint64_t>(k) * static_cast<uint64_t>(n) >= kStreamingMaxWeights) return false;
   if (m <= 16) return true;
   if (m > kStreamingMaxRows) return false;
   const long row_groups = s.row_groups;

@@ -696,7 +696,7 @@ int launch_skinny(const blkq4_gemm_args* a) {
 extern "C" int BLKQ4_SKINNY_ENTRY(const blkq4_gemm_args* a) {
   if (a->m < 1 || a->m > kStreamingMaxRows || (a->n % 16) != 0 || (a->k % 64) != 0) return static_cast<int>(hipErrorInvalidValue);
   // every offset is 32 bits wide: the packed weights (K N / 2 bytes) end below 4 GiB
-  if (static_cast<uint64_t>(a->k) * static_cast<uint64_t>(a->n) > kStreamingMaxWeights) return static_cast<int>(hipErrorInvalidValue);
+  if (static_cast<uint64_t>(a->k) * static_cast<uint64_t>(a->n) >= kStreamingMaxWeights) return static_cast<int>(hipErrorInvalidValue);
   if (!a->column_wise) {
     // blocks along N: a 16-column tile lies inside one block, and the meta data are fetched 16 bytes at a time
     if ((a->n % a->block_size) != 0 || (reinterpret_cast<uintptr_t>(a->scales) & 15u) != 0 ||

@@ -78,3 +78,27 @@ def test_plan_rejects_what_the_gemm_rejects(capi):
         with pytest.raises(capi.Blkq4Error) as e:
             capi.gemm_plan(*args)
         assert str(e.value) == message
+
+
+@pytest.mark.parametrize("m", [1, 4, 16, 64, 2048])
+def test_packed_weights_of_four_gib_and_more_are_refused_with_a_message(capi, m):
+    """every kernel addresses the packed weights with 32-bit byte offsets: k * n / 2 stays below 4 GiB"""
+    with pytest.raises(capi.Blkq4Error, match="must stay below 4 GiB"):
+        capi.gemm_plan(64, True, m, 131072, 65536)   # exactly 4 GiB
+    chosen, launched, text = capi.gemm_plan(64, True, m, 131072 - 32, 65536)
+    assert chosen == launched and chosen != 0, text
+
+
+def test_wide_layers_give_every_compute_unit_the_same_number_of_tiles(capi):
+    """five to sixteen rows, rows staged per slice: 4 to 7 column tiles per workgroup, no more workgroups than one round
+    of resident ones"""
+    import re
+    for m, k in ((16, 4096), (16, 8192), (8, 8192), (5, 11008), (4, 8192), (1, 11008)):
+        for n in (13312, 14336, 18432, 22016, 24576, 28672):
+            text = capi.gemm_plan(64, True, m, n, k)[2]
+            if not text.startswith("streaming:") or "rows staged per slice" not in text:
+                continue
+            tiles_per_workgroup = int(re.search(r"(\d+) column tile", text).group(1))
+            workgroups = int(re.search(r"(\d+) workgroups", text).group(1))
+            assert 4 <= tiles_per_workgroup <= 7 and workgroups <= 256, (m, n, k, text)
+            assert (n // 16 + tiles_per_workgroup - 1) // tiles_per_workgroup <= workgroups, (m, n, k, text)
