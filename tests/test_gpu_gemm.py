@@ -121,6 +121,8 @@ FIVE_TO_SEVEN_TILE_CASES = [
     (64, True, 4, 22016, 8192), (32, False, 2, 28672, 8256), (16, True, 3, 24576, 8192),
     # and a single row once K is longer than 8192
     (64, False, 1, 22016, 11008), (32, True, 1, 28672, 8320),
+    # six tiles with four waves: three workgroups per compute unit
+    (32, False, 7, 69664, 1088),
 ]
 
 
