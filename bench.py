@@ -599,7 +599,17 @@ def main(argv=None) -> int:
                    "checked": checked},
     }
     if "cpu_baseline" in head:
-        line["cpu_baseline"] = head["cpu_baseline"]
+        line["cpu_baseline"] = dict(head["cpu_baseline"])
+    # The metric has two halves (the M=2048 GEMM and the M=1 GEMV) and the configurations beside them: the
+    # objects a reader of this line is sure to keep whole carry all of them, compactly.
+    line["roofline"] = dict(head["roofline"])
+    line["roofline"]["kernel_us"] = head.get("kernel_us")
+    by_workload = {}
+    for key, res in results.items():
+        r = res.get("roofline")
+        if r is not None and key != "copy":
+            by_workload[key] = {"bound": r["bound"], "frac": r["frac"], "kernel_us": res["kernel_us"]}
+    line["roofline"]["by_workload"] = by_workload
     if "C2" in results:
         c2 = results["C2"]
         line["gemv"] = {"workload": c2["workload"], "value": c2["value"], "unit": "GB/s",
@@ -608,10 +618,21 @@ def main(argv=None) -> int:
                         "launches_per_timed_region": c2["launches_per_region"]}
         if "cpu_baseline" in c2:
             line["gemv"]["cpu_baseline"] = c2["cpu_baseline"]
+        line["roofline"]["gemv"] = {"workload": c2["workload"], "bound": "hbm", "achieved": c2["roofline"]["achieved"],
+                                    "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": c2["roofline"]["frac"],
+                                    "kernel_us": c2["kernel_us"], "traffic": c2["roofline"]["traffic"],
+                                    "weight_sets": c2["weight_sets"]}
+        if "cpu_baseline" in c2 and "cpu_baseline" in line:
+            line["cpu_baseline"]["gemv"] = {k: c2["cpu_baseline"][k] for k in ("value", "unit", "cores", "kind")}
     if not args.no_context:
         sys.stderr.write("[bench] context\n")
         line["context"] = bench_context(torch, capi, device, head_problem, args.steps, args.warmup)
-    line["all"] = results
+        for key, ctx in (("C4", "library_fp16_gemm_c4_shape"), ("C5", "library_fp16_gemm_c5_shape")):
+            if key in by_workload and ctx in line["context"]:
+                by_workload[key]["library_fp16_gemm_us"] = line["context"][ctx]["us"]
+    # the configurations the metric is defined on go last, so that they are what the end of the output shows
+    last = [k for k in ("C1", "C3", "C5_prepack", "C5", "C2", "C4") if k in results]
+    line["all"] = {k: results[k] for k in [k for k in results if k not in last] + last}
     print(json.dumps(line))
     if not parity_ok:
         sys.stderr.write("[bench] PARITY FAILED: " + json.dumps({k: v for k, v in checked.items() if not v["ok"]}) + "\n")

@@ -24,6 +24,9 @@ EXPORTED_SYMBOLS = (
     "blkq4_bf16_gemm_sm80",
     "blkq4_gemm_plan_sm80",
     "blkq4_fp16_gemm_noalloc_sm80",
+    "blkq4_fp16_gemm_noalloc_init_sm80",
+    "blkq4_gemm_workspace_info_sm80",
+    "blkq4_gemm_workspace_release_sm80",
     "blkq4_fp16_gemv_valu_sm80",
     "blkq4_error_message_create",
     "blkq4_error_message_cstr",
@@ -75,6 +78,13 @@ def load() -> ctypes.CDLL:
     u64p = ctypes.POINTER(ctypes.c_uint64)
     L.blkq4_gemm_plan_sm80.argtypes = [i, b, b, b, i, i, i, u64p, u64p, ctypes.c_char_p, sz, vp]
     L.blkq4_gemm_plan_sm80.restype = i
+    L.blkq4_fp16_gemm_noalloc_init_sm80.argtypes = [vp]
+    L.blkq4_fp16_gemm_noalloc_init_sm80.restype = i
+    ip = ctypes.POINTER(ctypes.c_int)
+    L.blkq4_gemm_workspace_info_sm80.argtypes = [vp, ip, ip, ip, ctypes.POINTER(sz), vp]
+    L.blkq4_gemm_workspace_info_sm80.restype = i
+    L.blkq4_gemm_workspace_release_sm80.argtypes = [vp]
+    L.blkq4_gemm_workspace_release_sm80.restype = i
     L.blkq4_error_message_create.restype = vp
     L.blkq4_error_message_cstr.argtypes = [vp]
     L.blkq4_error_message_cstr.restype = ctypes.c_char_p
@@ -209,3 +219,32 @@ def gemm_plan(block_size: int, column_wise: bool, m: int, n: int, k: int, has_of
                                 ctypes.byref(launched), text, len(text), err.h)
     _check(rc, err)
     return chosen.value, launched.value, text.value.decode()
+
+
+def noalloc_init():
+    """``blkq4_fp16_gemm_noalloc_init_sm80`` on the current device."""
+    L = load()
+    err = _ErrMsg(L)
+    _check(L.blkq4_fp16_gemm_noalloc_init_sm80(err.h), err)
+
+
+def workspace_info(stream=None):
+    """``blkq4_gemm_workspace_info_sm80`` -> (state, buffers_in_use, buffers_max, buffer_bytes); state 1: a GEMM
+    with a split plan issued on ``stream`` now has a workspace, 0: it would allocate one, -1: it would run the plan
+    that needs none."""
+    L = load()
+    err = _ErrMsg(L)
+    state, in_use, most = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    nbytes = ctypes.c_size_t(0)
+    rc = L.blkq4_gemm_workspace_info_sm80(_stream_ptr(stream), ctypes.byref(state), ctypes.byref(in_use),
+                                          ctypes.byref(most), ctypes.byref(nbytes), err.h)
+    _check(rc, err)
+    return state.value, in_use.value, most.value, nbytes.value
+
+
+def workspace_release():
+    """``blkq4_gemm_workspace_release_sm80``: frees every workspace (nothing that uses one may be running, queued or
+    replayed later)."""
+    L = load()
+    err = _ErrMsg(L)
+    _check(L.blkq4_gemm_workspace_release_sm80(err.h), err)

@@ -313,27 +313,28 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
     if (int code = blkq4_dev_gemv_dot(&args)) return device_failure(code, err);
     return 0;
   }
-  blkq4::Choice choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, blkq4_dev_workspace_capacity());
+  // The allocation-free entry point plans with what its buffer holds: a shape whose best plan would need more gets
+  // a smaller split or the unsplit kernel, never a refusal.
+  const size_t capacity = static_workspace ? blkq4_dev_static_workspace_capacity() : blkq4_dev_workspace_capacity();
+  blkq4::Choice choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, capacity);
   if (choice.family == blkq4::kFamilyTile && choice.t.split_k > 1) {
     void* workspace = nullptr;
     if (static_workspace) {
-      // the allocation-free entry point: the same plan, the workspace that lives in the library's device image
-      if (choice.t.workspace_bytes > blkq4_dev_static_workspace_capacity()) {
+      if (choice.t.workspace_bytes > capacity) {  // cannot happen: the plan was made for this capacity
         set_error(err, "Workspace of " + std::to_string(choice.t.workspace_bytes) +
-                           " bytes needed, the allocation-free entry point holds " +
-                           std::to_string(blkq4_dev_static_workspace_capacity()));
+                           " bytes needed, the allocation-free entry point holds " + std::to_string(capacity));
         return -1;
       }
       if (int code = blkq4_dev_static_workspace(&workspace)) return device_failure(code, err);
       args.workspace = workspace;
-      args.workspace_bytes = blkq4_dev_static_workspace_capacity();
+      args.workspace_bytes = capacity;
     } else {
       if (int code = blkq4_dev_workspace(stream, &workspace)) return device_failure(code, err);
       if (workspace == nullptr) {
         choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, 0);
       } else {
         args.workspace = workspace;
-        args.workspace_bytes = blkq4_dev_workspace_capacity();
+        args.workspace_bytes = capacity;
       }
     }
   }
@@ -488,6 +489,33 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
     text.copy(description, len);
     description[len] = '\0';
   }
+  return 0;
+}
+
+// Set-up of the allocation-free entry point on the current device: resolves the address of the workspace inside the
+// library's device image (which makes the runtime load that image, if it has not yet).
+extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_noalloc_init_sm80(void* err_msg_ptr) {
+  void* workspace = nullptr;
+  if (int code = blkq4_dev_static_workspace(&workspace)) return device_failure(code, static_cast<std::string*>(err_msg_ptr));
+  return 0;
+}
+
+// What a GEMM whose plan splits tiles would find on `stream` now (see the header).
+extern "C" BLKQ4_EXPORT int blkq4_gemm_workspace_info_sm80(void* stream, int* state, int* buffers_in_use,
+                                                           int* buffers_max, size_t* buffer_bytes, void* err_msg_ptr) {
+  int st = 0, in_use = 0, cap = 0;
+  if (int code = blkq4_dev_workspace_info(stream, &st, &in_use, &cap)) {
+    return device_failure(code, static_cast<std::string*>(err_msg_ptr));
+  }
+  if (state != nullptr) *state = st;
+  if (buffers_in_use != nullptr) *buffers_in_use = in_use;
+  if (buffers_max != nullptr) *buffers_max = cap;
+  if (buffer_bytes != nullptr) *buffer_bytes = blkq4_dev_workspace_capacity();
+  return 0;
+}
+
+extern "C" BLKQ4_EXPORT int blkq4_gemm_workspace_release_sm80(void* err_msg_ptr) {
+  if (int code = blkq4_dev_workspace_release()) return device_failure(code, static_cast<std::string*>(err_msg_ptr));
   return 0;
 }
 

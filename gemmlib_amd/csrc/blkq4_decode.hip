@@ -375,13 +375,13 @@ template <int BS, bool HAS_ZP, bool ROW, int R, int NT, int kWaves, int D>
 int launch_kernel(const blkq4_gemm_args* a) {
   const blkq4_decode_plan& p = a->decode;
   if (a->launched_id != nullptr) *a->launched_id = decode_id(ROW, R, NT, kWaves, D);
-  if (a->dry_run) return 0;
   const int slices = a->k / 128;
   const size_t lds = decode_lds_bytes(ROW, R, NT, kWaves, D);
   if (a->m > R || slices > kWaves * D || slices <= kWaves * (D - 1) || lds > kMaxLdsBytes || p.lds_bytes != lds ||
       p.grid != decode_grid(a->n, NT)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
+  if (a->dry_run) return 0;  // the plan has passed every check a launch makes
   constexpr auto kernel = decode_mfma_kernel<BS, HAS_ZP, R, NT, kWaves, D, ROW>;
   if (lds > 64 * 1024) {
     if (hipError_t e = raise_lds_limit<kernel>(); e != hipSuccess) return static_cast<int>(e);

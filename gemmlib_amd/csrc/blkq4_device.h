@@ -119,15 +119,21 @@ int blkq4_dev_gemv_dot(const blkq4_gemm_args* args);    /* fp16 GEMV on the vect
 int blkq4_dev_repack(const blkq4_repack_args* args);
 const char* blkq4_dev_error_string(int code);
 
-/* Workspace of the split tile kernels: the library-owned buffer of (current device, stream), allocated on first
- * use with a fixed size and its counters zeroed; *ptr = NULL (and 0 returned) when there is none and none can be
- * made (out of memory, or too many streams have one). */
+/* Workspace of the split tile kernels: the library-owned buffer of (current device, stream, the recording the
+ * stream is in, if any), allocated on first use with a fixed size and its counters zeroed; *ptr = NULL (and 0
+ * returned) when there is none and none can be made (out of memory, too many buffers handed out, or the stream is
+ * hipStreamPerThread). */
 size_t blkq4_dev_workspace_capacity(void);
 int blkq4_dev_workspace(void* stream, void** ptr);
+/* What a split GEMM issued on `stream` now would find: *state = 1 a buffer, 0 room to allocate one, -1 neither (it
+ * would run the unsplit plan); buffers handed out so far and the most there can be. */
+int blkq4_dev_workspace_info(void* stream, int* state, int* in_use, int* capacity);
+/* Frees every buffer (the caller promises that nothing that uses one is running, queued or will be replayed). */
+int blkq4_dev_workspace_release(void);
 /* The workspace inside the library's device image (nothing is ever allocated): one per device, shared by every
  * stream of that device. */
 size_t blkq4_dev_static_workspace_capacity(void);
-int blkq4_dev_static_workspace(void** ptr);
+int blkq4_dev_static_workspace(void** ptr);  /* resolves the buffer's address on the first call per device */
 
 #ifdef __cplusplus
 }

@@ -719,7 +719,6 @@ int launch_one(const blkq4_gemm_args* a) {
   const int n_tiles = (a->n + kBN - 1) / kBN;
   const int tiles = m_tiles * n_tiles;
   if (a->launched_id != nullptr) *a->launched_id = tile_id(RT, NT, WM, WN, PW, SK);
-  if (a->dry_run) return 0;
   int whole = tiles, split_tiles = 0, split_k = 1;
   float* partials = nullptr;
   int* counters = nullptr;
@@ -730,13 +729,18 @@ int launch_one(const blkq4_gemm_args* a) {
     whole = tiles - split_tiles;
     const size_t need = kCounterBytes + static_cast<size_t>(split_tiles) * split_k * BM * kBN * 4;
     if (split_tiles < 1 || split_tiles > tiles || split_k < 2 || split_k > a->k / kBK ||
-        static_cast<size_t>(split_tiles) * sizeof(int) > kCounterBytes || a->workspace == nullptr ||
-        a->workspace_bytes < need || (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
+        static_cast<size_t>(split_tiles) * sizeof(int) > kCounterBytes || t.workspace_bytes != need) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+    if (a->dry_run) return 0;  // the plan has passed every check a launch makes but those of the buffer itself
+    if (a->workspace == nullptr || a->workspace_bytes < need || (reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0) {
       return static_cast<int>(hipErrorInvalidValue);
     }
     counters = static_cast<int*>(a->workspace);
     partials = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + kCounterBytes);
   }
+  if (t.tiles != tiles) return static_cast<int>(hipErrorInvalidValue);
+  if (a->dry_run) return 0;
   const dim3 grid(static_cast<unsigned>(whole + split_tiles * split_k));
   // the launch's own status: a sticky error of an earlier, unrelated call stays where it is
   return static_cast<int>(launch_status(gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW, ROW, SK>, grid,

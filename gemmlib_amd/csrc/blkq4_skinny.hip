@@ -605,7 +605,6 @@ int launch_kernel(const blkq4_gemm_args* a) {
   static_assert(AM != kRowsPerSlotInLds || kPerSlotBytes <= kMaxLdsBytes, "slots do not fit in LDS");
   const bool refill = p.refill != 0;
   if (a->launched_id != nullptr) *a->launched_id = streaming_id(DEPTH, NT, MT, kWaves, AM, kSplit, refill);
-  if (a->dry_run) return 0;
   const size_t a_bytes = AM == kRowsWholeInLds ? ((((static_cast<size_t>(a->k) * 2) << p.rows_log2) + 1023) & ~size_t{1023})
                                                : kPerSlotBytes;
   constexpr int kGroupTiles = NT * (kWaves / kSplit);
@@ -618,6 +617,10 @@ int launch_kernel(const blkq4_gemm_args* a) {
       (kSplit == 1 && (reinterpret_cast<uintptr_t>(a->c) & 7u) != 0)) {
     return static_cast<int>(hipErrorInvalidValue);
   }
+  if constexpr (ROW && kWaves == 16) {
+    if (refill) return static_cast<int>(hipErrorInvalidValue);  // this kernel has no walking variant
+  }
+  if (a->dry_run) return 0;  // the plan has passed every check a launch makes
   auto launch = [&](auto* kernel, hipError_t attr) {
     if (attr != hipSuccess) return static_cast<int>(attr);
     // the launch's own status: a sticky error of an earlier, unrelated call stays where it is

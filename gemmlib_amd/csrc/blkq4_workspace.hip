@@ -1,11 +1,12 @@
 // Workspace of the split tile kernels (arrival counters + fp32 partial tiles): where it comes from.
 //
-//   blkq4_dev_workspace: one buffer per (device, stream), owned by the library, allocated on the first call
-//     that needs one and kept until the process ends.  Calls on one stream run in order, so they can share a
-//     buffer; calls on different streams may overlap, so they cannot.  A call that is being recorded into a graph
-//     may allocate too (the allocation is no stream operation; the thread's capture mode is set to relaxed around
-//     it, as tensor libraries do for their own allocations during capture).  A recorded call keeps using the
-//     buffer of the stream it was recorded on, whatever stream the graph is launched on later.
+//   blkq4_dev_workspace: buffers owned by the library, one per (device, stream, recording) -- see
+//     blkq4_workspace_table.h for why that is the key -- allocated by the first call that needs one and kept until
+//     blkq4_dev_workspace_release or the end of the process.  A call that is being recorded into a graph may
+//     allocate too (the allocation is no stream operation; the thread's capture mode is set to relaxed around it,
+//     as tensor libraries do for their own allocations during capture); the graph keeps using that buffer whatever
+//     stream it is launched on later, and nothing else ever uses it.  hipStreamPerThread names a different stream
+//     in every host thread, so the handle identifies nothing: such calls get no buffer (unsplit kernels).
 //
 //   blkq4_dev_static_workspace: a buffer inside the library's device image, for callers that must not allocate
 //     (code recorded into a graph by a harness that forbids it, tight serving loops).  Nothing is ever allocated;
@@ -24,11 +25,11 @@
 #include "blkq4_choose.h"
 #include "blkq4_device.h"
 #include "blkq4_launch.h"
+#include "blkq4_workspace_table.h"
 
 namespace {
 
 constexpr size_t kPoolBytes = blkq4::kCounterBytes + (size_t{32} << 20);
-constexpr int kMaxSlots = 16;  // streams with a buffer of their own; later ones run unsplit kernels
 constexpr size_t kStaticBytes = blkq4::kCounterBytes + (size_t{16} << 20);
 constexpr int kMaxDevices = 64;
 
@@ -41,14 +42,25 @@ __global__ void clear_counters(int* counters) {
   for (unsigned i = threadIdx.x; i < blkq4::kCounterBytes / sizeof(int); i += blockDim.x) counters[i] = 0;
 }
 
-struct Slot {
-  int device;
-  hipStream_t stream;
-  void* ptr;
-};
 std::mutex g_mutex;
-Slot g_slots[kMaxSlots];
-int g_slot_count = 0;
+blkq4::WorkspaceTable g_table;
+
+// (device, stream, recording) of a call on `stream` made now; false: calls on this stream get no buffer
+bool key_of(hipStream_t stream, blkq4::WorkspaceKey* key, hipError_t* error) {
+  *error = hipSuccess;
+  if (stream == hipStreamPerThread) return false;
+  int device = 0;
+  if ((*error = hipGetDevice(&device)) != hipSuccess) return false;
+  unsigned long long capture = 0;
+  if (stream != nullptr && stream != hipStreamLegacy) {  // the legacy default stream cannot record
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long id = 0;
+    if ((*error = hipStreamGetCaptureInfo(stream, &status, &id)) != hipSuccess) return false;
+    if (status == hipStreamCaptureStatusActive) capture = id + 1;  // never 0 for a recording
+  }
+  *key = blkq4::WorkspaceKey{device, stream, capture};
+  return true;
+}
 
 }  // namespace
 
@@ -56,25 +68,23 @@ extern "C" size_t blkq4_dev_workspace_capacity(void) { return kPoolBytes; }
 
 extern "C" int blkq4_dev_workspace(void* stream_ptr, void** ptr) {
   *ptr = nullptr;
-  hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
-  int device = 0;
-  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return static_cast<int>(e);
+  blkq4::WorkspaceKey key{};
+  hipError_t e = hipSuccess;
+  if (!key_of(static_cast<hipStream_t>(stream_ptr), &key, &e)) return static_cast<int>(e);
   std::lock_guard<std::mutex> lock(g_mutex);
-  for (int i = 0; i < g_slot_count; ++i) {
-    if (g_slots[i].device == device && g_slots[i].stream == stream) {
-      *ptr = g_slots[i].ptr;
-      return 0;
-    }
+  if (void* have = g_table.find(key)) {
+    *ptr = have;
+    return 0;
   }
-  if (g_slot_count == kMaxSlots) return 0;  // no workspace for this stream: unsplit kernels
+  if (!g_table.has_room(key.capture != 0)) return 0;  // no workspace for this call: unsplit kernels
   // An allocation is allowed while this or another thread records a graph only in relaxed mode.  The counters
   // are cleared on a stream of this function's own and waited for, so they are zero when this returns, whether
   // the caller's stream is executing or being recorded.
   hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
-  if (hipError_t e = hipThreadExchangeStreamCaptureMode(&mode); e != hipSuccess) return static_cast<int>(e);
+  if (e = hipThreadExchangeStreamCaptureMode(&mode); e != hipSuccess) return static_cast<int>(e);
   void* p = nullptr;
   hipStream_t own = nullptr;
-  hipError_t e = hipMalloc(&p, kPoolBytes);
+  e = hipMalloc(&p, kPoolBytes);
   if (e == hipSuccess) {
     e = hipStreamCreateWithFlags(&own, hipStreamNonBlocking);
     if (e == hipSuccess) {
@@ -90,9 +100,39 @@ extern "C" int blkq4_dev_workspace(void* stream_ptr, void** ptr) {
     return 0;
   }
   if (e != hipSuccess) return static_cast<int>(e);
-  g_slots[g_slot_count++] = Slot{device, stream, p};
+  g_table.add(key, p);
   *ptr = p;
   return 0;
+}
+
+// What a split GEMM issued on `stream` now would find: *state = 1 the call has a buffer, 0 it would allocate one,
+// -1 it would run the unsplit plan (no room for another buffer, or hipStreamPerThread).
+extern "C" int blkq4_dev_workspace_info(void* stream_ptr, int* state, int* in_use, int* capacity) {
+  blkq4::WorkspaceKey key{};
+  hipError_t e = hipSuccess;
+  const bool keyed = key_of(static_cast<hipStream_t>(stream_ptr), &key, &e);
+  if (e != hipSuccess) return static_cast<int>(e);
+  std::lock_guard<std::mutex> lock(g_mutex);
+  *state = !keyed ? -1 : g_table.find(key) != nullptr ? 1 : g_table.has_room(key.capture != 0) ? 0 : -1;
+  *in_use = g_table.in_use();
+  *capacity = blkq4::WorkspaceTable::capacity();
+  return 0;
+}
+
+// Frees every buffer.  The caller promises that no GEMM of this library is executing or queued and that no graph
+// holding one will be launched again.
+extern "C" int blkq4_dev_workspace_release(void) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  int current = 0;
+  hipError_t first = hipGetDevice(&current);
+  if (first != hipSuccess) return static_cast<int>(first);
+  g_table.release_all([&](int device, void* p) {
+    hipError_t e = hipSetDevice(device);
+    if (e == hipSuccess) e = hipFree(p);
+    if (e != hipSuccess && first == hipSuccess) first = e;
+  });
+  (void)hipSetDevice(current);
+  return static_cast<int>(first);
 }
 
 extern "C" size_t blkq4_dev_static_workspace_capacity(void) { return kStaticBytes; }

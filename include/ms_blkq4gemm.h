@@ -11,10 +11,30 @@
  *   - every pointer is DEVICE memory owned by the caller unless stated otherwise;
  *   - every `*_size` argument is a size in BYTES; the two outputs of the size query are ELEMENT counts;
  *   - `stream` is a hipStream_t cast to void* (nullptr = the default stream); calls are asynchronous
- *     with respect to that stream and allocate no device memory;
+ *     with respect to that stream;
  *   - `error_message` is nullptr or a `std::string*` that receives a message when the call fails;
  *   - the return value is 0 on success and -1 on failure; no exception crosses the boundary;
- *   - the library keeps no global state and may be called from several host threads.
+ *   - every entry point may be called from several host threads.
+ *
+ * Device memory and state.  The quantizer, the layout conversion and the queries allocate nothing and keep
+ * nothing.  The GEMM entry points keep ONE kind of state, which the reference's GEMM does not have
+ * (src/blkq4_f16_gemm_sm80.cu:38-153 allocates nothing): for some shapes (few tiles and a long K, e.g. m = 256,
+ * k = 11008, n = 4096) the fastest plan shares tiles out over several workgroups along K, and those leave fp32
+ * partial tiles in a workspace.  The first such call on a stream allocates that workspace with hipMalloc (32 MiB
+ * + 16 KiB; it waits for a small kernel on a stream of its own and, while a graph is being recorded, switches the
+ * calling thread's capture mode to relaxed around the allocation) and the library keeps it: one buffer per
+ * (device, stream handle, recording).  What follows from that:
+ *   - calls on different streams, and a recorded graph against eager calls or against another recorded graph,
+ *     never share a buffer and may run side by side;
+ *   - ONE recorded graph must not run twice at the same time (two executable copies of it launched on two
+ *     streams share the recording's buffer and would race);
+ *   - at most 16 streams and 16 recordings get a buffer; calls beyond that, calls on hipStreamPerThread and calls
+ *     made when the allocation fails run the best plan that needs no workspace (same results to the stated
+ *     tolerance, up to a quarter slower on the shapes above).  blkq4_gemm_workspace_info_sm80 tells which of the
+ *     two a call would get, blkq4_gemm_workspace_release_sm80 frees the buffers;
+ *   - blkq4_fp16_gemm_noalloc_sm80 is the GEMM that never allocates.
+ * Shapes whose plan does not split (all of the reference's own `m <= 16` cases, and most others) never touch any
+ * of this.
  *
  * The includer provides <cstdint> and <cstddef> (as with the reference header).
  */
@@ -164,17 +184,21 @@ int blkq4_bf16_gemm_sm80(
 
 /**
  * blkq4_fp16_gemm_sm80 for callers that cannot allocate device memory: code recorded into a graph by a harness
- * that forbids allocation, tight serving loops.  Same arguments, checks, messages, kernels and result bits as
- * blkq4_fp16_gemm_sm80.  The difference: when the chosen kernel splits tiles over K and needs a workspace for the
+ * that forbids allocation, tight serving loops.  Same arguments, checks and messages as blkq4_fp16_gemm_sm80 and
+ * every shape it takes.  The difference: when the chosen kernel splits tiles over K and needs a workspace for the
  * fp32 partial tiles, that workspace is a buffer inside the library's device image (16 MiB + 16 KiB per GPU, held
- * until the process ends) instead of the per-stream buffer blkq4_fp16_gemm_sm80 allocates on first use.  No
- * hipMalloc, hipFree or other allocating call is made.  A shape whose plan needs more than the buffer holds is
- * rejected with "Workspace of N bytes needed, the allocation-free entry point holds M" (-1); blkq4_fp16_gemm_sm80
- * takes such a shape.  All streams of a GPU share the one buffer: calls that overlap on one GPU race, so issue
- * them on one stream or order them yourself.
+ * until the process ends) instead of a buffer blkq4_fp16_gemm_sm80 allocates on first use, and the plan is made for
+ * that size: a shape whose fastest plan needs more (m = 300, n = 28672, k = 4096 wants 30 MiB) runs a smaller
+ * split or the unsplit kernel, so its result can differ from blkq4_fp16_gemm_sm80's in the last bit (another
+ * order of summation) while shapes whose plan fits give the same bits.  No hipMalloc, hipFree or other allocating
+ * call is made.  All streams of a GPU share the one buffer: calls that overlap on one GPU race, so issue them on
+ * one stream or order them yourself.  The first call on a device asks the runtime for the buffer's address, which
+ * makes it load the library's device image if nothing has yet: call blkq4_fp16_gemm_noalloc_init_sm80 (or this
+ * entry point once) on each device before recording a graph.
  *
  * No counterpart in the reference (whose GEMM needs no workspace): it is for the callers that cannot allocate.
  */
+int blkq4_fp16_gemm_noalloc_init_sm80(void* error_message);
 int blkq4_fp16_gemm_noalloc_sm80(
   int block_size,
   bool column_wise_blocking,
@@ -194,8 +218,8 @@ int blkq4_fp16_gemm_noalloc_sm80(
  * accumulation and single rounding of the output; other shapes are rejected (-1).
  *
  * No counterpart in the reference (whose small-M kernel, src/mickey/blk_q4/f16_gemm_sm80.h:63-72, uses tensor
- * cores too).  blkq4_fp16_gemm_sm80 picks between this form and the MFMA form by shape; this entry point runs this
- * form whatever the shape, so that the two can be measured against each other.
+ * cores too).  blkq4_fp16_gemm_sm80 runs this form for no shape (its MFMA kernels are faster on every shape
+ * measured); it is reachable by this name only, so that the two forms can be measured against each other.
  */
 int blkq4_fp16_gemv_valu_sm80(
   int block_size,
@@ -230,6 +254,27 @@ int blkq4_gemm_plan_sm80(
     uint64_t* launched_id,
     char* description, size_t description_size,
     void* error_message);
+
+/**
+ * The workspaces of the GEMM's split plans (see "Device memory and state" at the top).  Host-side bookkeeping; no
+ * kernel is launched.
+ *   blkq4_gemm_workspace_info_sm80: *state = 1 when a GEMM issued on `stream` now (in the recording the stream is
+ *     in, if any) has a workspace already, 0 when it would allocate one on first need, -1 when it would run the
+ *     plan without a workspace (all buffers handed out, or hipStreamPerThread); buffers handed out so far, the
+ *     most there can be, and the size of one.  Any of the outputs may be null.
+ *   blkq4_gemm_workspace_release_sm80: frees every buffer.  The caller promises that no GEMM of this library is
+ *     running or queued and that no graph recorded with one will be launched again.
+ *
+ * No counterpart in the reference, whose GEMM has no workspace.
+ */
+int blkq4_gemm_workspace_info_sm80(
+    void* stream,
+    int* state,
+    int* buffers_in_use,
+    int* buffers_max,
+    size_t* buffer_bytes,
+    void* error_message);
+int blkq4_gemm_workspace_release_sm80(void* error_message);
 
 /**
  * Helpers for callers that cannot construct a C++ std::string (ctypes, cgo, JNI ...): create an

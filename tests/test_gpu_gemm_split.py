@@ -131,3 +131,61 @@ def test_split_tiles_recorded_on_a_stream_of_their_own_and_on_two_streams_at_onc
     torch.cuda.synchronize()
     assert torch.equal(o1.view(torch.int16), eager.view(torch.int16))
     assert torch.equal(o2.view(torch.int16), eager.view(torch.int16))
+
+
+def test_a_recording_has_a_workspace_of_its_own_and_the_thread_stream_has_none(oracle, capi, device):
+    """Which calls share a workspace (the promises of the public header): eager calls on a stream share one; a
+    recording on that same stream gets another, so the graph may run on any stream while the recording stream
+    works eagerly; a second recording gets a third; hipStreamPerThread gets none and runs the unsplit plan."""
+    bs, m, n, k = 64, 200, 5120, 8192
+    _assert_split_plan(capi, bs, True, m, n, k, "128 x 128", 3)
+    a, w = gaussian_problem(123, m, n, k)
+    a2, _ = gaussian_problem(124, m, n, k)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, w, True)
+    a_dev, a2_dev = to_dev(a, device), to_dev(a2, device)
+    want = torch.empty(m, n, dtype=torch.float16, device=device)
+    want2 = torch.empty_like(want)
+    s, t = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        capi.gemm(bs, True, m, n, k, a_dev, q_w, q_s, q_zp, want)
+        capi.gemm(bs, True, m, n, k, a2_dev, q_w, q_s, q_zp, want2)
+    torch.cuda.synchronize()
+    state, in_use, most, nbytes = capi.workspace_info(s)
+    assert state == 1 and 1 <= in_use <= most == 32 and nbytes == (32 << 20) + (16 << 10)
+    graphs, outs = [], []
+    for i in range(2):
+        out = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(s):
+            with torch.cuda.graph(g, stream=s):
+                before = capi.workspace_info(s)
+                capi.gemm(bs, True, m, n, k, a_dev, q_w, q_s, q_zp, out)
+                after = capi.workspace_info(s)
+        assert before[0] == 0 and after[0] == 1 and after[1] == before[1] + 1, (before, after)
+        graphs.append(g)
+        outs.append(out)
+    assert capi.workspace_info(s)[:2] == (1, in_use + 2)   # eager calls on s still have theirs
+    # both graphs on t and on the legacy stream while s works eagerly on other data
+    eager_out = torch.empty_like(want)
+    for rep in range(5):
+        with torch.cuda.stream(t):
+            graphs[0].replay()
+        graphs[1].replay()
+        with torch.cuda.stream(s):
+            capi.gemm(bs, True, m, n, k, a2_dev, q_w, q_s, q_zp, eager_out)
+        torch.cuda.synchronize()
+        for out in outs:
+            assert torch.equal(out.view(torch.int16), want.view(torch.int16)), rep
+            out.fill_(float("nan"))
+        assert torch.equal(eager_out.view(torch.int16), want2.view(torch.int16)), rep
+    # hipStreamPerThread (the handle 2): no workspace, the plan that needs none, same result within tolerance
+    assert capi.workspace_info(2)[0] == -1
+    out = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+    capi.gemm(bs, True, m, n, k, a_dev, q_w, q_s, q_zp, out, stream=2)
+    torch.cuda.synchronize()
+    assert capi.workspace_info(2)[:2] == (-1, in_use + 2)
+    assert max_rel_err(to_np(out), to_np(want)) <= 1e-2 and not torch.isnan(out).any()
+    canon, sc, z = oracle.quantize(bs, True, w, True)
+    rows = np.arange(0, m, 25)
+    ref = oracle.gemm(np.ascontiguousarray(a[rows]), oracle.dequantize(bs, True, canon, sc, z))
+    assert max_rel_err(to_np(out)[rows], ref) <= 1e-2
