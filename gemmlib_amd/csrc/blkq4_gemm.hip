@@ -754,7 +754,7 @@ int launch_one(const blkq4_gemm_args* a) {
 
 // The tile shapes that exist, (RT, NT, WM, WN, PW): what blkq4::choose() may ask for.  Those with whole rows
 // of 32 or 64 (one row tile only) have no split form and no form for blocks along N.
-#define BLKQ4_TILE_SHAPES(X) X(8, 2, 1, 4, 0) X(4, 2, 1, 4, 4) X(4, 1, 1, 4, 4) X(2, 1, 1, 4, 4)
+#define BLKQ4_TILE_SHAPES(X) X(8, 2, 1, 4, 0) X(8, 1, 1, 4, 4) X(4, 2, 1, 4, 4) X(4, 1, 1, 4, 4) X(2, 1, 1, 4, 4)
 #define BLKQ4_TILE_SHAPES_ONE_ROW_TILE(X) X(1, 1, 1, 4, 4) X(1, 1, 1, 8, 0) X(2, 1, 1, 8, 0)
 
 template <int BS, bool HAS_ZP>
