@@ -12,6 +12,7 @@ needed to build.
 from __future__ import annotations
 
 import argparse
+import json
 import os
 import subprocess
 import sys
@@ -28,26 +29,21 @@ LIB_PATH = os.path.join(LIB_DIR, "libms_blkq4gemm.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-HIP_SOURCES = ["blkq4_prepack.hip", "blkq4_skinny.hip", "blkq4_skinny_bf16.hip", "blkq4_gemm.hip", "blkq4_gemm_bf16.hip",
-               "blkq4_workspace.hip", "blkq4_gemv.hip", "blkq4_decode.hip", "blkq4_decode_bf16.hip"]
-# Kernel arguments of the decode kernels arrive in registers with the wave (the code object keeps a prologue that
-# loads them for firmware that does not preload).
-EXTRA_HIP_FLAGS = {
-    "blkq4_decode.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
-    "blkq4_decode_bf16.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
-}
-HOST_SOURCES = ["blkq4_api.cpp"]
-
-# -ffp-contract=off: every fused multiply-add the quantizer needs is written as an explicit fmaf.
-# The division stays IEEE correctly rounded (hipcc's default); no fast-math anywhere.
-# packed-fp32-ops is switched off for the device code (the host pass prints a harmless warning).
-HIP_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
-    "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-fast-math",
-    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function", "-Wno-pass-failed",
-]
-HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wextra", "-D_GLIBCXX_USE_CXX11_ABI=1"]
+# Sources and flags come from csrc/build_manifest.json, which CMakeLists.txt reads too.
+#   -ffp-contract=off: every fused multiply-add the quantizer needs is written as an explicit fmaf.
+#   The division stays IEEE correctly rounded; no fast-math anywhere.
+#   packed-fp32-ops is switched off for the device code (the host pass prints a harmless warning).
+#   Kernel arguments of the decode kernels arrive in registers with the wave (the code object keeps a prologue that
+#   loads them for firmware that does not preload).
+with open(os.path.join(CSRC, "build_manifest.json")) as _f:
+    MANIFEST = json.load(_f)
+HIP_SOURCES = list(MANIFEST["hip_sources"])
+HOST_SOURCES = list(MANIFEST["host_sources"])
+EXTRA_HIP_FLAGS = {k: list(v) for k, v in MANIFEST["extra_hip_flags"].items()}
+HIP_FLAGS = ["--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fvisibility=hidden", *MANIFEST["hip_flags"]]
+for _feature in MANIFEST["hip_target_features_off"]:
+    HIP_FLAGS += ["-Xclang", "-target-feature", "-Xclang", "-" + _feature]
+HOST_FLAGS = ["-std=c++17", "-fPIC", "-fvisibility=hidden", *MANIFEST["host_flags"]]
 
 
 def _run(cmd, quiet_stderr_filter=None):
