@@ -19,6 +19,7 @@ EXPORTED_SYMBOLS = (
     "blkq4_fp16_gemm_bias_sm80",
     "blkq4_fp16_quant_sm80",
     "blkq4_fp16_quant_size_sm80",
+    "blkq4_fp16_quant_selfcheck_sm80",
     "blkq4_fp16_repack_sm80",
     "blkq4_bf16_quant_sm80",
     "blkq4_bf16_gemm_sm80",
@@ -69,6 +70,8 @@ def load() -> ctypes.CDLL:
     # `int64_t&` is a pointer at the ABI level
     L.blkq4_fp16_quant_size_sm80.argtypes = [i, b, i, i, i64p, i64p, vp]
     L.blkq4_fp16_quant_size_sm80.restype = i
+    L.blkq4_fp16_quant_selfcheck_sm80.argtypes = [vp, vp, sz, vp]
+    L.blkq4_fp16_quant_selfcheck_sm80.restype = i
     L.blkq4_fp16_repack_sm80.argtypes = [i, i, i, vp, vp, sz, vp, sz, vp]
     L.blkq4_fp16_repack_sm80.restype = i
     L.blkq4_bf16_quant_sm80.argtypes = L.blkq4_fp16_quant_sm80.argtypes
@@ -248,3 +251,11 @@ def workspace_release():
     L = load()
     err = _ErrMsg(L)
     _check(L.blkq4_gemm_workspace_release_sm80(err.h), err)
+
+
+def quant_selfcheck(counts, stream=None):
+    """``blkq4_fp16_quant_selfcheck_sm80``: ``counts`` is a device tensor of four int64 (disagreements for asymmetric
+    blocks, symmetric blocks, the rounding; cases looked at)."""
+    L = load()
+    err = _ErrMsg(L)
+    _check(L.blkq4_fp16_quant_selfcheck_sm80(_stream_ptr(stream), _ptr(counts), _nbytes(counts), err.h), err)

@@ -519,6 +519,19 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_workspace_release_sm80(void* err_msg_ptr)
   return 0;
 }
 
+// The fp16 quantizer computes its divisions and its rounding with sequences shorter than the IEEE ones; this runs
+// the comparison of the two over the whole domain on the current GPU (see the header).
+extern "C" BLKQ4_EXPORT int blkq4_fp16_quant_selfcheck_sm80(void* stream, void* counts, size_t counts_size,
+                                                            void* err_msg_ptr) {
+  auto* err = static_cast<std::string*>(err_msg_ptr);
+  if (counts == nullptr || counts_size != 4 * sizeof(uint64_t) || (reinterpret_cast<uintptr_t>(counts) & 7u) != 0) {
+    set_error(err, "Unexpected counter buffer: four 64-bit counters in device memory, 8-byte aligned, expected");
+    return -1;
+  }
+  if (int code = blkq4_dev_quant_selfcheck(counts, stream)) return device_failure(code, err);
+  return 0;
+}
+
 extern "C" BLKQ4_EXPORT int blkq4_fp16_repack_sm80(int to_sm80, int rows, int columns, void* stream,
                                                    void const* src, size_t src_size, void* dst,
                                                    size_t dst_size, void* err_msg_ptr) {

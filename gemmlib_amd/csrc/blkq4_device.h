@@ -117,6 +117,9 @@ int blkq4_dev_decode(const blkq4_gemm_args* args);      /* decode kernel: few ro
 int blkq4_dev_decode_bf16(const blkq4_gemm_args* args); /* the same with bf16 a, scales, c and bias */
 int blkq4_dev_gemv_dot(const blkq4_gemm_args* args);    /* fp16 GEMV on the vector ALU (no MFMA): 1 <= m <= 4, blocks along K */
 int blkq4_dev_repack(const blkq4_repack_args* args);
+/* The fp16 quantizer's shortened arithmetic against its IEEE definition over the whole domain; counts: four
+ * 64-bit counters in device memory (disagreements of asymmetric blocks, symmetric blocks, the rounding; cases). */
+int blkq4_dev_quant_selfcheck(void* counts, void* stream);
 const char* blkq4_dev_error_string(int code);
 
 /* Workspace of the split tile kernels: the library-owned buffer of (current device, stream, the recording the

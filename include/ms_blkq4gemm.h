@@ -148,6 +148,19 @@ int blkq4_fp16_repack_sm80(
     void* error_message);
 
 /**
+ * Self-check of blkq4_fp16_quant_sm80's arithmetic on the GPU it runs on.  The quantizer is bound by its vector
+ * instructions, so it computes the reference's two divisions (src/mickey/blk_q4/f16_quant_sm80.cuh:104-112, :294)
+ * and its roundf (:110, :298) with shorter instruction sequences than the IEEE ones.  This entry point compares
+ * the short forms with the IEEE forms over their WHOLE domain -- every range an fp16 block can have (about 10^9 pairs),
+ * every nonzero symmetric extreme, every float in [0, 15] -- and leaves four 64-bit counters in `counts` (device memory,
+ * counts_size = 32): disagreements for asymmetric blocks, for symmetric blocks, for the rounding (all three must
+ * be 0), and the number of cases looked at.  A few milliseconds; asynchronous like every other call.
+ *
+ * No counterpart in the reference.
+ */
+int blkq4_fp16_quant_selfcheck_sm80(void* stream, void* counts, size_t counts_size, void* error_message);
+
+/**
  * bf16: the quantizer and the GEMM above for bf16 weights, activations, scales, bias and output, the
  * element type the reference's templates anticipate (reference: src/mickey/blk_q4/f16_quant_sm80.cuh:16,
  * src/mickey/cutlass_ext/q4gemm/warp/quantb_mma_tensor_op.h:95-114) and its entry points reject

@@ -165,3 +165,17 @@ def test_benchmark_config_shapes(oracle, capi, device, name):
     w_t = (torch.randn(columns, rows, generator=g, dtype=torch.float32) * 0.02).to(torch.float16)
     w = w_t.view(torch.int16).numpy().view(np.float16)
     check_against_oracle(oracle, capi, device, bs, w, has_offsets)
+
+
+def test_shortened_quantizer_arithmetic_equals_the_ieee_form_over_its_whole_domain(capi, device):
+    """blkq4_fp16_quant_selfcheck_sm80: the fp16 quantizer's short division sequences and its one-instruction
+    rounding against the IEEE forms of the reference's arithmetic (src/mickey/blk_q4/f16_quant_sm80.cuh:96-122,
+    :291-298) for every range a block can have, every nonzero symmetric extreme and every float in [0, 15], on this GPU."""
+    counts = torch.full((4,), -1, dtype=torch.int64, device=device)
+    capi.quant_selfcheck(counts)
+    torch.cuda.synchronize()
+    asym, sym, rounding, cases = counts.cpu().tolist()
+    assert (asym, sym, rounding) == (0, 0, 0)
+    assert cases == 31745 * 31744 + (2 * 31744 - 2) + 0x41700000 + 1
+    with pytest.raises(capi.Blkq4Error, match="Unexpected counter buffer"):
+        capi.quant_selfcheck(counts[:3])
