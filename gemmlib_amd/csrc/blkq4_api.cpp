@@ -479,7 +479,8 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
     } else {
       const auto& t = choice.t;
       text = "tile: " + std::to_string(32 * t.rt * t.wm) + " x " + std::to_string(32 * t.nt * t.wn) + ", " +
-             std::to_string(t.wm * t.wn) + " + " + std::to_string(t.pw) + " waves, " + std::to_string(t.tiles) + " tiles";
+             std::to_string(t.wm * t.wn * t.kw) + " + " + std::to_string(t.pw) + " waves" +
+             (t.kw > 1 ? " (the computing waves split the k tile)" : "") + ", " + std::to_string(t.tiles) + " tiles";
       if (t.split_k > 1) {
         text += ", the last " + std::to_string(t.split_tiles) + " in " + std::to_string(t.split_k) + " parts (workspace " +
                 std::to_string(t.workspace_bytes) + " bytes)";

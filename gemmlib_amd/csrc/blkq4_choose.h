@@ -47,10 +47,10 @@ inline uint64_t streaming_id(int depth, int nt, int mt, int waves, int am, int s
          static_cast<uint64_t>(mt) << 24 | static_cast<uint64_t>(waves) << 16 | static_cast<uint64_t>(am) << 12 |
          static_cast<uint64_t>(split) << 4 | (refill ? 1u : 0u);
 }
-inline uint64_t tile_id(int rt, int nt, int wm, int wn, int pw, bool split) {
+inline uint64_t tile_id(int rt, int nt, int wm, int wn, int pw, bool split, int kw = 1) {
   return 2ull << 60 | static_cast<uint64_t>(rt) << 40 | static_cast<uint64_t>(nt) << 32 |
          static_cast<uint64_t>(wm) << 24 | static_cast<uint64_t>(wn) << 16 | static_cast<uint64_t>(pw) << 8 |
-         (split ? 1u : 0u);
+         static_cast<uint64_t>(kw) << 4 | (split ? 1u : 0u);
 }
 // the GEMV without MFMA (blkq4_gemv.hip; run only when asked for by name): rows kept (1, 2 or 4) and waves of a
 // workgroup
@@ -71,7 +71,7 @@ inline uint64_t choice_id(const Choice& c) {
   if (c.family == kFamilyDecode) return decode_id(c.d.row != 0, c.d.rows, c.d.nt, c.d.waves, c.d.depth);
   return c.family == kFamilyStreaming
              ? streaming_id(c.s.depth, c.s.nt, c.s.mt, c.s.waves, c.s.am, c.s.split, c.s.refill != 0)
-             : tile_id(c.t.rt, c.t.nt, c.t.wm, c.t.wn, c.t.pw, c.t.split_k > 1);
+             : tile_id(c.t.rt, c.t.nt, c.t.wm, c.t.wn, c.t.pw, c.t.split_k > 1, c.t.kw);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -465,12 +465,24 @@ inline double tile_round_us(const TileShape& t, int k_tiles, long busy) {
   return c.fixed + k_tiles * (c.step_idle + (b > c.flat_until ? (b - c.flat_until) * c.step_slope : 0.0));
 }
 
+// Tiles of 128 x 32 whose four computing waves split the k tile (kw = 4): only when one round of them covers the
+// problem.  Fitted to measurements with 256 of them on the chip (fp16, blocks of 64, N = 4096 or 8192): K = 2048 10.3 us,
+// 4096 16.4 - 16.9, 6144 24.7, 8192 30.2 -- 3.2 us outside the main loop (the sum of the four waves' accumulators
+// through LDS is part of it) and 0.215 us per 64-deep k tile.  Against the other plans' estimates that hands them
+// M = 129 ... 256 at N = 4096 up to K of about 5000 (same process, M = 256, K = N = 4096: 16.5 us against 19.0 in 64 x 128
+// tiles, 17.8 with those split in two along K, 17.5 streaming; K = 6144: 24.7 against 23.4 split, which keeps it).
+inline double k_split_waves_estimate_us(const TileShape& t, int k) {
+  (void)t;
+  return 3.2 + (k / 64) * 0.215;
+}
+
 // Estimated time of the tile kernel with shape t (split or not) on k: whole rounds of unsplit tiles, a last
 // round of what is left of them, then one round of parts: their share of the k tiles, the partial tile
 // written once and all parts read by the workgroup that arrives last (about 100 GB/s) plus 4 us for the cache
 // write-back and invalidate and the two extra barriers (measured: 64 x 128 in 2 parts 17.7 - 19.1 us against
 // 18.7 unsplit at M = 256, K = N = 4096; 128 x 128 in 3 parts 32.7 against 44.6 us at K = 11008).
 inline double tile_estimate_us(const TileShape& t, int k) {
+  if (t.kw > 1) return k_split_waves_estimate_us(t, k);
   const int kt = k / 64;
   const long whole = t.tiles - (t.split_k > 1 ? t.split_tiles : 0);
   double us = static_cast<double>(whole / kComputeUnits) * tile_round_us(t, kt, kComputeUnits);
@@ -515,6 +527,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
   auto shape = [&](int rt, int nt, int wm, int wn, int pw) {
     TileShape t{};
     t.rt = rt; t.nt = nt; t.wm = wm; t.wn = wn; t.pw = pw;
+    t.kw = 1;
     t.split_k = 1;
     t.tiles = static_cast<int>(ceil_div(m, 32 * rt * wm) * ceil_div(n, 32 * nt * wn));
     return t;
@@ -535,6 +548,19 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
     }
   }
   best_unsplit_us = best_us;
+  if (column_wise) {
+    // 128 x 32 tiles of four waves that split the k tile, when one round of them covers the problem
+    TileShape t = shape(4, 1, 1, 1, 4);
+    t.kw = 4;
+    if (t.tiles <= kComputeUnits) {
+      const double us = k_split_waves_estimate_us(t, k);
+      if (us < best_us) {
+        best = t;
+        best_us = us;
+        best_unsplit_us = us;
+      }
+    }
+  }
   for (const auto& sh : kTileShapes) {
     TileShape t = shape(sh[0], sh[1], sh[2], sh[3], sh[4]);
     const int rem = t.tiles % kComputeUnits;

@@ -60,10 +60,13 @@ typedef struct {
 } blkq4_streaming_plan;
 
 /* Which tile kernel runs: wm x wn computing waves of (32 rt) x (32 nt) outputs, pw producer waves.
+ * kw = 4 (with wm = wn = 1): four computing waves share the one (32 rt) x (32 nt) tile and split every 64-deep k tile
+ * between them; kw = 1 otherwise.
  * split_k > 1: the last split_tiles tiles of the tile order are computed by split_k workgroups each, which
  * leave fp32 partial tiles in the workspace; the last of them to finish sums them in a fixed order. */
 typedef struct {
   int rt, nt, wm, wn, pw;
+  int kw;
   int split_k;            /* 1: no workspace needed */
   int split_tiles;        /* 0 without a split */
   int tiles;              /* all tiles of the problem */

@@ -94,7 +94,7 @@ constexpr int stage_slot(int g, int u, int pairs, int slots) {
 // ROW: quantization blocks run along N (one k, BS columns).  The scales and zero-points of a k tile are
 // then, per group of BS columns, 64 consecutive rows in the packed order described in blkq4_device.h:
 // 128 + 64 bytes, copied as they are.
-template <int BS, int RT, int NT, int WM, int WN, int PW, bool ROW>
+template <int BS, int RT, int NT, int WM, int WN, int PW, bool ROW, int KW = 1>
 struct Stage {
   static constexpr int kCopiers = (PW > 0) ? PW : WM * WN;     // waves that share out the copies of a stage
   static constexpr int kBlocks = kBK / BS;                     // quantization block rows per k tile
@@ -120,7 +120,7 @@ struct Stage {
   // for the small ones (0.3 us).  Eight slots for those: M = 300, K = N = 4096 21.2 -> 18.8 us, M = 64, N = 18432 23.3 ->
   // 19.6, M = 256 19.0 -> 18.3, M = 512 (256 workgroups: bound by what L2 delivers) 23.6 -> 23.2.  Six slots for the
   // 128 x 128 tiles change nothing (+- 2 %), eight for the 256-column tiles of one row tile lose 5 %.
-  static constexpr bool kDeep = PW > 0 && RT * NT <= 2;
+  static constexpr bool kDeep = PW > 0 && (RT * NT <= 2 || KW > 1);  // (waves that split the k tile: 8 MFMAs or fewer per tile)
   static constexpr int kStages = (kDeep && 8 * kBytes <= 160 * 1024) ? 8 : (4 * kBytes <= 160 * 1024) ? 4 : 3;
   static constexpr int kDistance = kStages - 1;  // the slot being refilled is the one nobody reads
   static_assert((kDistance - 1) * kOps <= 63, "more copies in flight than the counter holds");
@@ -132,18 +132,29 @@ struct Stage {
 // leaves its fp32 partial tile in `partials` and counts itself in the tile's arrival counter; the one that
 // arrives last adds the parts up in the order 0, 1, ..., split_k - 1 (so the result does not depend on who
 // that is), clears the counter for the next launch and runs the epilogue.  Nobody waits for anybody.
-template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW, bool SK, bool BF = kBF>
-__global__ __launch_bounds__(64 * (WM * WN + PW))
-    __attribute__((amdgpu_waves_per_eu((WM * WN + PW) / 4, (WM * WN + PW) / 4))) void gemm_mfma_kernel(
+// KW = 4: the four computing waves share ONE (32*RT) x (32*NT) tile and split every 64-deep k tile between them, wave w
+// owning its 16-deep step w (WM = WN = 1).  A weight fragment is then converted once per RT MFMAs whatever the
+// tile's width, which is what small problems need: with tiles of 128 x 32 every compute unit of the chip has a tile at
+// M = 256, N = 4096 and converts 3.25 instructions' worth per MFMA, where 64 x 128 tiles of four 64 x 32 waves convert
+// 6.5 and occupy half the chip (same process: 16.5 against 19.0 us, 17.8 with those tiles split in two along K).  The
+// waves' accumulators are added up through LDS in the epilogue, in wave order.  (Tiles of 128 x 64 of this kind were
+// measured too and are not built: 20.8 us on that problem and no problem found where they are ahead.)
+template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW, bool SK, int KW = 1, bool BF = kBF>
+__global__ __launch_bounds__(64 * (WM * WN * KW + PW))
+    __attribute__((amdgpu_waves_per_eu((WM * WN * KW + PW) / 4, (WM * WN * KW + PW) / 4))) void gemm_mfma_kernel(
         const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ S,
         const uint8_t* __restrict__ Z, uint16_t* __restrict__ C, const uint16_t* __restrict__ bias, int M, int N,
         int K, int m_tiles, int whole_tiles, int split_tiles, int split_k, float* __restrict__ partials,
         int* __restrict__ counters) {
-  using St = Stage<BS, RT, NT, WM, WN, PW, ROW>;
-  constexpr int kComputeWaves = WM * WN;
+  using St = Stage<BS, RT, NT, WM, WN, PW, ROW, KW>;
+  constexpr int kComputeWaves = WM * WN * KW;
+  constexpr bool KS = KW > 1;
+  constexpr int kAhead = KS ? 2 : 1;
+  static_assert(KW == 1 || (KW == 4 && WM == 1 && WN == 1 && PW > 0 && !ROW && !SK),
+                "waves that split the k tile: four of them, one tile, producer waves, blocks along K, no split tiles");
   static_assert(!ROW || St::kGroups % 2 == 0, "scale copies take two column groups at a time");
   constexpr int kCopiers = St::kCopiers;
-  static_assert((WM * WN + PW) % 4 == 0, "whole waves per SIMD");
+  static_assert((WM * WN * KW + PW) % 4 == 0, "whole waves per SIMD");
   constexpr int kBlocks = St::kBlocks;
   constexpr int kOps = St::kOps;
   constexpr int kStages = St::kStages;
@@ -161,8 +172,8 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = (wave / WN) % WM;  // position of the wave's tile inside the workgroup tile
-  const int wn = wave % WN;
+  const int wm = KS ? 0 : (wave / WN) % WM;  // position of the wave's tile inside the workgroup tile
+  const int wn = KS ? 0 : wave % WN;
   const int cw = (PW > 0) ? max(wave - kComputeWaves, 0) : wave;  // index among the copying waves
   const int lane = tid & 63;
   const int i = lane & 31;  // row of an activation fragment / column of a weight fragment
@@ -295,13 +306,17 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
 #pragma unroll
       for (int q = 0; q < kOps; ++q) BLKQ4_COPY_OP(q, min(s, KT - 1), s);
     }
-    wait_vmcnt<(kDistance - 1) * kOps>();
+    // kAhead: how many tiles past the one being multiplied the computing waves read after a tile's barrier (the
+    // waves that split the k tile read two ahead: their tile is short, and a read issued behind the barrier would be
+    // needed before it can have arrived)
+    static_assert(kDistance - 1 - kAhead >= 0, "the ring is too short for reading that far ahead");
+    wait_vmcnt<(kDistance - kAhead) * kOps>();
     block_barrier();
     for (int kt = 0; kt < KT; ++kt) {
-      // tile kt+1 must have landed: everything but the kDistance-2 newest groups (near the end
+      // tile kt+kAhead must have landed: everything but the kDistance-1-kAhead newest groups (near the end
       // fewer groups than that are in flight, then wait for all of them)
       if (kt + kDistance <= KT) {
-        wait_vmcnt<(kDistance - 2) * kOps>();
+        wait_vmcnt<(kDistance - 1 - kAhead) * kOps>();
       } else {
         wait_vmcnt<0>();
       }
@@ -463,7 +478,7 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   Bf16Consts bdc[NT][kMeta], bndc[NT][kMeta];  // bf16: these instead
   uint4 mrow_s[2][NT][2], mrow_z[2][NT];  // blocks along N: meta of 16-row groups 2h (steps 0, 1) and 2h + 1 (steps 2, 3)
 
-  {
+  if constexpr (!KS) {
     const uint32_t s0 = 0;
     BLKQ4_READ_B(words, dc, s0);
     BLKQ4_READ_ROW_META(0, s0);
@@ -474,6 +489,109 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
     for (int x = 0; x < 4 * NT; ++x) {
       BLKQ4_PIECE(0, words, 0, dc, 0, x);
     }
+  }
+
+  if constexpr (KS) {
+    // ---- waves that split the k tile ----
+    // Wave `wave` owns the 16-deep step `wave` of every k tile: the activation fragments of that step, word `wave`
+    // of every lane's packed unit, the scale and zero-point of the block that word lies in.  One barrier per k
+    // tile, as in the other loop: it publishes tile kt + 1 and retires the slot of tile kt - 1.  Behind it the
+    // wave reads tile kt + 1 from LDS and converts its weights in the shadow of tile kt's MFMAs.
+    const uint32_t ks_a_rd = lds0 + static_cast<uint32_t>(i) * 128u + (((4 * h + wave) ^ ((i >> 1) & 7)) * 16u);
+    const uint32_t ks_w_rd = lds0 + St::kABytes + lane * 16 + 4 * wave;
+    const int ks_blk = (BS == 64) ? 0 : (BS == 32) ? h : (2 * h + (wave >> 1));
+    const uint32_t ks_m_rd = lds0 + St::kABytes + St::kBBytes + ks_blk * 256 + i;
+    // Two tiles are read ahead: behind the barrier of tile kt the wave asks LDS for tile kt + 2 (fragments into one of
+    // four buffers, packed words and scales into one of two), converts tile kt + 1 from what it asked for a tile ago,
+    // and multiplies tile kt.
+    uint32_t kw_words[2][NT][1];
+    uint32_t kw_sc[2][NT], kw_zp[2][NT];
+    DequantConsts kdc[NT][1];
+    Bf16Consts bkdc[NT][1];
+    half8_t kaf[4][RT];
+#define BLKQ4_KS_READ(abuf_, wbuf_, so_)                                                               \
+  {                                                                                                    \
+    _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                                   \
+      kw_words[wbuf_][t][0] = lds_read_u32((so_) + ks_w_rd, t * 1024);                                 \
+      kw_sc[wbuf_][t] = lds_read_u16((so_) + ks_m_rd + i, t * 128);                                    \
+      kw_zp[wbuf_][t] = HAS_ZP ? lds_read_u8((so_) + ks_m_rd, t * 128 + 64) : 8u;                      \
+    }                                                                                                  \
+    _Pragma("unroll") for (int r = 0; r < RT; ++r) kaf[abuf_][r] = as_half8(lds_read_16((so_) + ks_a_rd, r * 4096)); \
+  }
+#define BLKQ4_KS_CONSTS(wbuf_)                                                                         \
+  _Pragma("unroll") for (int t = 0; t < NT; ++t) {                                                     \
+    if constexpr (kBF) {                                                                               \
+      bkdc[t][0] = make_bf16_consts(kw_sc[wbuf_][t], kw_zp[wbuf_][t]);                                 \
+    } else {                                                                                           \
+      kdc[t][0] = make_dequant_consts(kw_sc[wbuf_][t], kw_zp[wbuf_][t]);                               \
+    }                                                                                                  \
+  }
+    // MFMA slot behind which pair g2 (of 2 * NT) of the next tile's fragments is converted: spread over the tile
+    auto ks_pair_slot = [](int g2) constexpr { return g2 * kMfmas / (2 * NT); };
+    BLKQ4_KS_READ(0, 0, 0u);
+    BLKQ4_KS_CONSTS(0);
+#pragma unroll
+    for (int x = 0; x < 4 * NT; ++x) {
+      BLKQ4_PIECE(0, kw_words[0], 0, kdc, 0, x);
+    }
+    BLKQ4_KS_READ(1, 1, static_cast<uint32_t>(St::kBytes));
+    auto ks_tile = [&](const uint32_t sn2, auto cur_tag) __attribute__((always_inline)) {
+      constexpr int cur = decltype(cur_tag)::value;  // tile kt modulo 4
+      constexpr int wcur = cur & 1, wnext = 1 - wcur;
+      block_barrier();
+      BLKQ4_KS_READ((cur + 2) & 3, wcur, sn2);
+      BLKQ4_PIN();
+      BLKQ4_KS_CONSTS(wnext);
+      half8_t wf_[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) wf_[t] = BLKQ4_WFRAG(wcur, t);
+#pragma unroll
+      for (int r = 0; r < RT; ++r) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const int x_ = r * NT + t;
+          if constexpr (kBF) {
+            acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wf_[t]),
+                                                               __builtin_bit_cast(bf16x8_t, kaf[cur][r]), acc[r][t], 0, 0, 0);
+          } else {
+            acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[t], kaf[cur][r], acc[r][t], 0, 0, 0);
+          }
+#pragma unroll
+          for (int g2 = 0; g2 < 2 * NT; ++g2) {
+            if (ks_pair_slot(g2) == x_) {
+              BLKQ4_PIECE_AO(kw_words[wnext], 0, 2 * g2);
+              BLKQ4_PIECE_AO(kw_words[wnext], 0, 2 * g2 + 1);
+              BLKQ4_PIECE_PA(kdc, 0, 0, 2 * g2);
+              BLKQ4_PIECE_PA(kdc, 0, 0, 2 * g2 + 1);
+              BLKQ4_PIECE_PM(wnext, kdc, 0, 0, 2 * g2);
+              BLKQ4_PIECE_PM(wnext, kdc, 0, 0, 2 * g2 + 1);
+            }
+          }
+          BLKQ4_PIN();
+        }
+      }
+    };
+    // ring slot of tile kt + 2, as a byte offset; four tiles per trip so that the register buffers are constants
+    uint32_t sn2 = (2 % kStages) * St::kBytes;
+    auto advance = [&]() { sn2 = (sn2 + St::kBytes == kStages * St::kBytes) ? 0u : sn2 + St::kBytes; };
+    for (int kt = 0; kt < KT; kt += 4) {
+      ks_tile(sn2, std::integral_constant<int, 0>{});
+      advance();
+      if (kt + 1 < KT) {
+        ks_tile(sn2, std::integral_constant<int, 1>{});
+        advance();
+      }
+      if (kt + 2 < KT) {
+        ks_tile(sn2, std::integral_constant<int, 2>{});
+        advance();
+      }
+      if (kt + 3 < KT) {
+        ks_tile(sn2, std::integral_constant<int, 3>{});
+        advance();
+      }
+    }
+#undef BLKQ4_KS_READ
+#undef BLKQ4_KS_CONSTS
   }
 
   // One 16-deep k step: RT*NT MFMAs on fragment buffers `cur_`; in their shadow the LDS reads of the
@@ -562,7 +680,7 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
       }
     }
   };
-  for (int kt0 = 0; kt0 < KT; kt0 += kStages) {
+  for (int kt0 = 0; !KS && kt0 < KT; kt0 += kStages) {
     k_tile(kt0, std::integral_constant<int, 0>{});
     if (kt0 + 1 < KT) k_tile(kt0 + 1, std::integral_constant<int, 1>{});
     if (kt0 + 2 < KT) k_tile(kt0 + 2, std::integral_constant<int, 2>{});
@@ -667,7 +785,57 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
       }
     }
   }
-  {
+  if constexpr (KS) {
+    // The four waves' accumulators as fp32 tiles [wave][row][32 * NT columns + 4 of padding] in the (by now unused)
+    // ring; then all 256 threads add them up in wave order, 8 columns per thread, and store whole rows.
+    constexpr int kRowWords = 32 * NT + 4;  // rows start 4 banks apart: 16 lanes write, or read, all 64 banks once
+    constexpr uint32_t kPartBytes = 32 * RT * kRowWords * 4;
+    static_assert(KW * kPartBytes <= kStages * St::kBytes, "the waves' partial tiles do not fit in the ring");
+    const uint32_t mine = lds0 + static_cast<uint32_t>(wave) * kPartBytes + static_cast<uint32_t>(i * kRowWords + 4 * h) * 4u;
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const float e0 = acc[r][t][4 * g], e1 = acc[r][t][4 * g + 1], e2 = acc[r][t][4 * g + 2], e3 = acc[r][t][4 * g + 3];
+          lds_write_16(mine, (32 * r * kRowWords + 32 * t + 8 * g) * 4, __float_as_uint(e0), __float_as_uint(e1),
+                       __float_as_uint(e2), __float_as_uint(e3));
+        }
+    block_barrier();
+    constexpr int kChunks = 4 * NT;              // 16-byte chunks of a row of the output tile
+    constexpr int kRowsPerPass = 256 / kChunks;  // all 256 threads of the computing waves
+    const int chunk = tid % kChunks, srow = tid / kChunks;
+    const int col = nw0 + chunk * 8;
+    uint4 bias8 = make_uint4(0, 0, 0, 0);
+    if (bias != nullptr && col < N) bias8 = *reinterpret_cast<const uint4*>(bias + col);
+    const uint32_t rd = lds0 + static_cast<uint32_t>(srow * kRowWords + chunk * 8) * 4u;
+#pragma unroll
+    for (int it = 0; it < 32 * RT / kRowsPerPass; ++it) {
+      float sum[8];
+#pragma unroll
+      for (int p = 0; p < KW; ++p) {
+        const uint4 lo = lds_read_16(rd, p * kPartBytes + it * kRowsPerPass * kRowWords * 4);
+        const uint4 hi = lds_read_16(rd, p * kPartBytes + it * kRowsPerPass * kRowWords * 4 + 16);
+        const float v[8] = {__uint_as_float(lo.x), __uint_as_float(lo.y), __uint_as_float(lo.z), __uint_as_float(lo.w),
+                            __uint_as_float(hi.x), __uint_as_float(hi.y), __uint_as_float(hi.z), __uint_as_float(hi.w)};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum[e] = (p == 0) ? v[e] : sum[e] + v[e];
+      }
+      uint4 v = make_uint4(float_to_bits<kBF>(sum[0]) | (float_to_bits<kBF>(sum[1]) << 16),
+                           float_to_bits<kBF>(sum[2]) | (float_to_bits<kBF>(sum[3]) << 16),
+                           float_to_bits<kBF>(sum[4]) | (float_to_bits<kBF>(sum[5]) << 16),
+                           float_to_bits<kBF>(sum[6]) | (float_to_bits<kBF>(sum[7]) << 16));
+      if (bias != nullptr) {
+        v = make_uint4(add_bias_pair_t<kBF>(v.x, bias8.x), add_bias_pair_t<kBF>(v.y, bias8.y),
+                       add_bias_pair_t<kBF>(v.z, bias8.z), add_bias_pair_t<kBF>(v.w, bias8.w));
+      }
+      const int m = m0 + it * kRowsPerPass + srow;
+      if (m < M && col < N) {
+        __builtin_nontemporal_store(uint4_t{v.x, v.y, v.z, v.w}, reinterpret_cast<uint4_t*>(C + static_cast<size_t>(m) * N + col));
+      }
+    }
+  } else {
     constexpr int kRowBytes = 64 * NT + 16;        // padded: consecutive rows start 4 (NT=2: 36) banks apart
     constexpr int kPassTiles = (RT < 4) ? RT : 4;  // row tiles staged at a time
     constexpr int kChunks = 4 * NT;                // 16-byte chunks per row
@@ -710,7 +878,7 @@ __global__ __launch_bounds__(64 * (WM * WN + PW))
   }
 }
 
-template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW, bool SK>
+template <int BS, bool HAS_ZP, int RT, int NT, int WM, int WN, int PW, bool ROW, bool SK, int KW = 1>
 int launch_one(const blkq4_gemm_args* a) {
   constexpr int BM = 32 * RT * WM;
   constexpr int kBN = 32 * NT * WN;
@@ -718,7 +886,7 @@ int launch_one(const blkq4_gemm_args* a) {
   const int m_tiles = (a->m + BM - 1) / BM;
   const int n_tiles = (a->n + kBN - 1) / kBN;
   const int tiles = m_tiles * n_tiles;
-  if (a->launched_id != nullptr) *a->launched_id = tile_id(RT, NT, WM, WN, PW, SK);
+  if (a->launched_id != nullptr) *a->launched_id = tile_id(RT, NT, WM, WN, PW, SK, KW);
   int whole = tiles, split_tiles = 0, split_k = 1;
   float* partials = nullptr;
   int* counters = nullptr;
@@ -743,8 +911,8 @@ int launch_one(const blkq4_gemm_args* a) {
   if (a->dry_run) return 0;
   const dim3 grid(static_cast<unsigned>(whole + split_tiles * split_k));
   // the launch's own status: a sticky error of an earlier, unrelated call stays where it is
-  return static_cast<int>(launch_status(gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW, ROW, SK>, grid,
-                                        dim3(64 * (WM * WN + PW)), 0, a->stream, static_cast<const uint8_t*>(a->a),
+  return static_cast<int>(launch_status(gemm_mfma_kernel<BS, HAS_ZP, RT, NT, WM, WN, PW, ROW, SK, KW>, grid,
+                                        dim3(64 * (WM * WN * KW + PW)), 0, a->stream, static_cast<const uint8_t*>(a->a),
                                         static_cast<const uint8_t*>(a->packed_w),
                                         static_cast<const uint8_t*>(a->scales),
                                         static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c),
@@ -756,11 +924,21 @@ int launch_one(const blkq4_gemm_args* a) {
 // of 32 or 64 (one row tile only) have no split form and no form for blocks along N.
 #define BLKQ4_TILE_SHAPES(X) X(8, 2, 1, 4, 0) X(8, 1, 1, 4, 4) X(4, 2, 1, 4, 4) X(4, 1, 1, 4, 4) X(2, 1, 1, 4, 4)
 #define BLKQ4_TILE_SHAPES_ONE_ROW_TILE(X) X(1, 1, 1, 4, 4) X(1, 1, 1, 8, 0) X(2, 1, 1, 8, 0)
+// (RT, NT) of the tiles whose four computing waves split the k tile (one tile per workgroup, four producer waves);
+// blocks along K, no split form
+#define BLKQ4_TILE_SHAPES_K_SPLIT_WAVES(X) X(4, 1)
 
 template <int BS, bool HAS_ZP>
 int launch_plan(const blkq4_gemm_args* a) {
   const blkq4_tile_plan& t = a->tile;
   const bool sk = t.split_k > 1;
+#define BLKQ4_TRY(RT_, NT_)                                                                            \
+  if (t.kw == 4 && t.rt == RT_ && t.nt == NT_ && t.wm == 1 && t.wn == 1 && t.pw == 4 && a->column_wise && !sk) { \
+    return launch_one<BS, HAS_ZP, RT_, NT_, 1, 1, 4, false, false, 4>(a);                               \
+  }
+  BLKQ4_TILE_SHAPES_K_SPLIT_WAVES(BLKQ4_TRY)
+#undef BLKQ4_TRY
+  if (t.kw != 1) return static_cast<int>(hipErrorInvalidValue);
 #define BLKQ4_TRY(RT_, NT_, WM_, WN_, PW_)                                                              \
   if (t.rt == RT_ && t.nt == NT_ && t.wm == WM_ && t.wn == WN_ && t.pw == PW_) {                        \
     if (a->column_wise) {                                                                               \

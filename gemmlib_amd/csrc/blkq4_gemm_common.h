@@ -44,6 +44,14 @@ __device__ __forceinline__ uint32_t lds_read_u16(uint32_t addr, int imm = 0) {
 __device__ __forceinline__ uint32_t lds_read_u8(uint32_t addr, int imm = 0) {
   return *(reinterpret_cast<const __attribute__((address_space(3))) uint8_t*>(addr) + imm);
 }
+__device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr, int imm = 0) {
+  const auto* p = reinterpret_cast<const __attribute__((address_space(3))) uint8_t*>(addr) + imm;
+  return *reinterpret_cast<const __attribute__((address_space(3))) uint32_t*>(p);
+}
+__device__ __forceinline__ void lds_write_16(uint32_t addr, int imm, uint32_t x, uint32_t y, uint32_t z, uint32_t w) {
+  auto* p = reinterpret_cast<__attribute__((address_space(3))) uint8_t*>(addr) + imm;
+  *reinterpret_cast<__attribute__((address_space(3))) lds_u32x4_t*>(p) = lds_u32x4_t{x, y, z, w};
+}
 typedef uint32_t lds_u32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ void lds_write_8(uint32_t addr, int imm, uint32_t lo, uint32_t hi) {
   auto* p = reinterpret_cast<__attribute__((address_space(3))) uint8_t*>(addr) + imm;

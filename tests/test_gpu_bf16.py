@@ -152,6 +152,8 @@ EXACT_CASES = [
     (64, True, 768, 1056, 576), (16, True, 129, 1056, 576),
     # five to seven column tiles per workgroup (wide layers, rows staged per slice)
     (64, True, 16, 18432, 1088), (32, False, 9, 22016, 1088), (16, True, 12, 28672, 1216), (32, True, 16, 57344, 1024),
+    # 128 x 32 tiles whose four computing waves split the k tile
+    (64, False, 255, 4096, 3008), (16, True, 200, 4096, 4096),
 ]
 
 

@@ -126,7 +126,35 @@ FIVE_TO_SEVEN_TILE_CASES = [
 ]
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + SMALL_TILE_CASES + WIDE_TILE32_CASES + LONG_K_CASES + VERY_WIDE_CASES + SIX_AND_EIGHT_TILE_CASES + FIVE_TO_SEVEN_TILE_CASES)
+# 128 x 32 tiles whose four computing waves split the k tile (one round of them covers the problem): a whole number of
+# trips through the unrolled loop and not (K = 3008 is 47 k tiles), rows past M in the last tile, every block size
+K_SPLIT_WAVES_CASES = [
+    (64, True, 256, 4096, 4096), (64, False, 255, 4096, 3008), (32, True, 256, 4096, 2112), (16, True, 200, 4096, 4096),
+]
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", K_SPLIT_WAVES_CASES)
+def test_k_split_waves_cases_run_the_tile_they_are_meant_for(capi, bs, has_offsets, m, n, k):
+    for bf16 in (False, True):
+        text = capi.gemm_plan(bs, True, m, n, k, has_offsets, bf16)[2]
+        assert text.startswith("tile: 128 x 32, 4 + 4 waves (the computing waves split the k tile)"), text
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", K_SPLIT_WAVES_CASES[:2])
+def test_k_split_waves_on_gaussian_data_and_with_bias(oracle, capi, device, bs, has_offsets, m, n, k):
+    got, q_w, q_s, q_zp, a = run_gaussian(oracle, capi, device, bs, has_offsets, m, n, k, seed=3000 + m + k, sample_rows=40)
+    # every call the same bits (the four waves' sums are added in wave order), and the bias as a separate add would
+    bias = (torch.randn(n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.float16)
+    fused = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+    capi.gemm(bs, True, m, n, k, to_dev(a, device), q_w, q_s, q_zp, fused, bias=bias.to(device))
+    torch.cuda.synchronize()
+    again = gemm_on_gpu(capi, device, bs, a, q_w, q_s, q_zp, n)
+    assert np.array_equal(again.view(np.uint16), got.view(np.uint16))
+    want = (torch.from_numpy(got.view(np.int16).copy()).view(torch.float16) + bias).view(torch.int16).numpy()
+    assert np.array_equal(fused.cpu().view(torch.int16).numpy(), want)
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", REFERENCE_CASES + EXTRA_CASES + K_SPLIT_WAVES_CASES + EDGE_CASES + WIDE_SKINNY_CASES + LARGE_TILE_CASES + SMALL_TILE_CASES + WIDE_TILE32_CASES + LONG_K_CASES + VERY_WIDE_CASES + SIX_AND_EIGHT_TILE_CASES + FIVE_TO_SEVEN_TILE_CASES)
 def test_exact_on_reference_construction(oracle, capi, device, bs, has_offsets, m, n, k):
     run_kat(oracle, capi, device, bs, has_offsets, m, n, k)
 
