@@ -554,10 +554,9 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
     t.kw = 4;
     if (t.tiles <= kComputeUnits) {
       const double us = k_split_waves_estimate_us(t, k);
-      if (us < best_us) {
+      if (us < best_us) {  // (the bar a split plan has to clear stays that of the other unsplit shapes)
         best = t;
         best_us = us;
-        best_unsplit_us = us;
       }
     }
   }

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 # (block_size, column_wise, has_offsets, m, n, k, tile the plan must name, parts)
 SPLIT_CASES = [
     (64, True, True, 100, 5120, 5120, "64 x 128", 3),
-    (32, True, False, 256, 4096, 4096, "64 x 128", 2),
+    (32, True, False, 256, 3072, 4096, "64 x 128", 2),
     (64, True, True, 200, 5120, 8192, "128 x 128", 3),
     (16, True, True, 65, 8192, 5120, "128 x 128", 4),
     (64, True, False, 300, 28672, 4096, "128 x 256", 3),
