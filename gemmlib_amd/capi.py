@@ -24,6 +24,7 @@ EXPORTED_SYMBOLS = (
     "blkq4_bf16_quant_sm80",
     "blkq4_bf16_gemm_sm80",
     "blkq4_gemm_plan_sm80",
+    "blkq4_gemm_with_plan_sm80",
     "blkq4_fp16_gemm_noalloc_sm80",
     "blkq4_fp16_gemm_noalloc_init_sm80",
     "blkq4_gemm_workspace_info_sm80",
@@ -88,6 +89,8 @@ def load() -> ctypes.CDLL:
     L.blkq4_gemm_workspace_info_sm80.restype = i
     L.blkq4_gemm_workspace_release_sm80.argtypes = [vp]
     L.blkq4_gemm_workspace_release_sm80.restype = i
+    L.blkq4_gemm_with_plan_sm80.argtypes = [ctypes.c_char_p, i, b, b, i, i, i, vp, vp, sz, vp, sz, vp, sz, vp, sz, vp, sz, vp]
+    L.blkq4_gemm_with_plan_sm80.restype = i
     L.blkq4_error_message_create.restype = vp
     L.blkq4_error_message_cstr.argtypes = [vp]
     L.blkq4_error_message_cstr.restype = ctypes.c_char_p
@@ -259,3 +262,15 @@ def quant_selfcheck(counts, stream=None):
     L = load()
     err = _ErrMsg(L)
     _check(L.blkq4_fp16_quant_selfcheck_sm80(_stream_ptr(stream), _ptr(counts), _nbytes(counts), err.h), err)
+
+
+def gemm_with_plan(plan: str, block_size: int, column_wise: bool, m: int, n: int, k: int, a, q_weights, q_scales, q_zp, out,
+                   stream=None, bf16=False):
+    """``blkq4_gemm_with_plan_sm80``: the GEMM with the kernel and its shape given as text (``"auto"``, ``"tile ..."``,
+    ``"streaming ..."``, ``"decode ..."``) instead of the cost model's choice."""
+    L = load()
+    err = _ErrMsg(L)
+    rc = L.blkq4_gemm_with_plan_sm80(plan.encode(), block_size, column_wise, bf16, m, n, k, _stream_ptr(stream), _ptr(a),
+                                     _nbytes(a), _ptr(q_weights), _nbytes(q_weights), _ptr(q_scales), _nbytes(q_scales),
+                                     _ptr(q_zp), _nbytes(q_zp), _ptr(out), _nbytes(out), err.h)
+    _check(rc, err)

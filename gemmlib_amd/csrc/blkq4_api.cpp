@@ -7,6 +7,8 @@
 #include "ms_blkq4gemm.h"
 
 #include <cstdint>
+#include <cstdio>
+#include <cstring>
 #include <string>
 
 #include "blkq4_choose.h"
@@ -196,13 +198,84 @@ int launch_choice(const blkq4::Choice& choice, bool bf16, const blkq4_gemm_args*
               : (streaming ? blkq4_dev_skinny(args) : blkq4_dev_gemm(args));
 }
 
+// A plan given as text (blkq4_gemm_with_plan_sm80): the kernel family and its shape parameters, everything else
+// derived the way blkq4::choose() derives it.  Whether such a kernel exists and fits the problem is the launchers'
+// check.  Returns false and says why when the text is no plan.
+bool parse_plan(const char* text, bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity,
+                blkq4::Choice* c, std::string* why) {
+  *c = blkq4::Choice{};
+  int v[7] = {0, 0, 0, 0, 0, 0, 0};
+  if (text == nullptr || std::strcmp(text, "auto") == 0) {
+    *c = blkq4::choose(column_wise, bf16, m, n, k, workspace_capacity);
+    return true;
+  }
+  if (std::sscanf(text, "tile %d %d %d %d %d %d %d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5], &v[6]) == 7) {
+    auto& t = c->t;
+    c->family = blkq4::kFamilyTile;
+    t.rt = v[0]; t.nt = v[1]; t.wm = v[2]; t.wn = v[3]; t.pw = v[4]; t.kw = v[5];
+    if (t.rt < 1 || t.nt < 1 || t.wm < 1 || t.wn < 1 || t.pw < 0 || t.kw < 1 || v[6] < 1 || t.rt * t.wm > 64 || t.nt * t.wn > 64) {
+      *why = "tile RT NT WM WN PW KW PARTS: positive numbers (PW may be 0, PARTS 1 means no split)";
+      return false;
+    }
+    t.tiles = static_cast<int>(blkq4::ceil_div(m, 32 * t.rt * t.wm) * blkq4::ceil_div(n, 32 * t.nt * t.wn));
+    t.split_k = v[6];
+    if (t.split_k > 1) {
+      // the tiles of the last, partly filled round (all of them when there is one round only), as choose() splits
+      t.split_tiles = t.tiles % blkq4::kComputeUnits ? t.tiles % blkq4::kComputeUnits : t.tiles;
+      t.workspace_bytes = blkq4::tile_workspace_bytes(t);
+      if (t.workspace_bytes > workspace_capacity || static_cast<size_t>(t.split_tiles) * sizeof(int) > blkq4::kCounterBytes) {
+        *why = "the split needs a workspace of " + std::to_string(t.workspace_bytes) + " bytes, more than there is";
+        return false;
+      }
+    }
+    return true;
+  }
+  if (std::sscanf(text, "streaming %d %d %d %d %d %d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5]) == 6) {
+    if (m > blkq4::kStreamingMaxRows || v[0] < 1 || v[1] < 1 || (v[2] != 1 && v[2] != 2) || v[3] < 1 || v[3] > 16 ||
+        (v[4] != blkq4::kRowsWholeInLds && v[4] != blkq4::kRowsPerSlotInLds) || (v[5] != 1 && v[5] != v[3]) ||
+        (v[2] == 1 && m > 16)) {
+      *why = "streaming DEPTH NT MT WAVES ROWS SPLIT: MT 1 (up to 16 rows) or 2 (row groups of 32), ROWS 1 (whole in LDS) or 2 "
+             "(staged per slice), SPLIT = WAVES (the waves split K) or 1; at most 1024 rows";
+      return false;
+    }
+    auto& p = c->s;
+    c->family = blkq4::kFamilyStreaming;
+    p.depth = v[0]; p.nt = v[1]; p.mt = v[2]; p.waves = v[3]; p.am = v[4]; p.split = v[5];
+    if (p.mt == 2) {
+      p.rows_log2 = 5;
+      p.row_groups = (m + 31) / 32;
+    } else {
+      p.row_groups = 1;
+      while ((1 << p.rows_log2) < m) ++p.rows_log2;
+    }
+    blkq4::streaming_geometry(&p, !column_wise, n, k);
+    return true;
+  }
+  if (std::sscanf(text, "decode %d %d %d %d", &v[0], &v[1], &v[2], &v[3]) == 4) {
+    if (v[0] < 1 || v[0] > blkq4::kDecodeMaxRows || v[1] < 1 || v[1] > 8 || v[2] < 1 || v[2] > 16 || v[3] < 1 || v[3] > 16 ||
+        (n % 16) != 0) {
+      *why = "decode ROWS NT WAVES DEPTH: rows kept (a power of two, at least m), column tiles per workgroup, waves, slices per wave";
+      return false;
+    }
+    auto& d = c->d;
+    c->family = blkq4::kFamilyDecode;
+    d.row = column_wise ? 0 : 1;
+    d.rows = v[0]; d.nt = v[1]; d.waves = v[2]; d.depth = v[3];
+    d.grid = blkq4::decode_grid(n, d.nt);
+    d.lds_bytes = static_cast<uint32_t>(blkq4::decode_lds_bytes(d.row != 0, d.rows, d.nt, d.waves, d.depth));
+    return true;
+  }
+  *why = "a plan is \"auto\", \"tile RT NT WM WN PW KW PARTS\", \"streaming DEPTH NT MT WAVES ROWS SPLIT\" or \"decode ROWS NT WAVES DEPTH\"";
+  return false;
+}
+
 // reference: src/blkq4_f16_gemm_sm80.cu:319-429 and :38-153 (blkq4_gemm_sm80_T); bias_ptr == nullptr or
 // bias_size == 0: no bias
 int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int n, int k, void* stream, void const* act_ptr,
                size_t a_size, void const* weights_ptr, size_t weights_size, void const* scales_ptr,
                size_t scales_size, void const* offsets_ptr, size_t offsets_size, void const* bias_ptr,
                size_t bias_size, void* output_ptr, size_t output_size, void* err_msg_ptr,
-               bool static_workspace = false, bool valu_gemv = false) {
+               bool static_workspace = false, bool valu_gemv = false, const char* plan = nullptr) {
   auto* err = static_cast<std::string*>(err_msg_ptr);
   if (!supported_block_size(block_size)) {
     set_error(err, "Unsupported block size: " + std::to_string(block_size));
@@ -316,7 +389,17 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
   // The allocation-free entry point plans with what its buffer holds: a shape whose best plan would need more gets
   // a smaller split or the unsplit kernel, never a refusal.
   const size_t capacity = static_workspace ? blkq4_dev_static_workspace_capacity() : blkq4_dev_workspace_capacity();
-  blkq4::Choice choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, capacity);
+  blkq4::Choice choice;
+  if (plan != nullptr) {
+    // a plan given by the caller (blkq4_gemm_with_plan_sm80)
+    std::string why;
+    if (!parse_plan(plan, column_wise_blocking, bf16, m, n, k, capacity, &choice, &why)) {
+      set_error(err, "Unknown plan: " + why);
+      return -1;
+    }
+  } else {
+    choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, capacity);
+  }
   if (choice.family == blkq4::kFamilyTile && choice.t.split_k > 1) {
     void* workspace = nullptr;
     if (static_workspace) {
@@ -331,6 +414,10 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
     } else {
       if (int code = blkq4_dev_workspace(stream, &workspace)) return device_failure(code, err);
       if (workspace == nullptr) {
+        if (plan != nullptr && std::strcmp(plan, "auto") != 0) {
+          set_error(err, "No workspace for the split the plan asks for (blkq4_gemm_workspace_info_sm80 says why)");
+          return -1;
+        }
         choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, 0);
       } else {
         args.workspace = workspace;
@@ -499,6 +586,18 @@ extern "C" BLKQ4_EXPORT int blkq4_fp16_gemm_noalloc_init_sm80(void* err_msg_ptr)
   void* workspace = nullptr;
   if (int code = blkq4_dev_static_workspace(&workspace)) return device_failure(code, static_cast<std::string*>(err_msg_ptr));
   return 0;
+}
+
+// The GEMM with the kernel and its shape given by the caller instead of the cost model (see the header): what the
+// model's choices are measured against.
+extern "C" BLKQ4_EXPORT int blkq4_gemm_with_plan_sm80(const char* plan, int block_size, bool column_wise_blocking, bool bf16,
+                                                      int m, int n, int k, void* stream, void const* act_ptr, size_t a_size,
+                                                      void const* weights_ptr, size_t weights_size, void const* scales_ptr,
+                                                      size_t scales_size, void const* offsets_ptr, size_t offsets_size,
+                                                      void* output_ptr, size_t output_size, void* err_msg_ptr) {
+  return gemm_entry(bf16, block_size, column_wise_blocking, m, n, k, stream, act_ptr, a_size, weights_ptr, weights_size,
+                    scales_ptr, scales_size, offsets_ptr, offsets_size, nullptr, 0, output_ptr, output_size, err_msg_ptr,
+                    /*static_workspace=*/false, /*valu_gemv=*/false, plan != nullptr ? plan : "auto");
 }
 
 // What a GEMM whose plan splits tiles would find on `stream` now (see the header).

@@ -334,7 +334,15 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
     // splitting waves' rings hold, which then ask for a fifth more slices than there are (K = 5120,
     // N = 13824: 14.5 -> 12.7 us).  Four slices in flight per wave: with eight the kernel needs 90 registers
     // and a SIMD holds five waves instead of seven (52 against 55 us at N = 128256).
-    const size_t max_row_bytes = (row ? 32 : 16) * 1024;
+    // (blocks along N with more than four rows: whatever fits, one or two workgroups per compute unit -- M = 16, K = 4096,
+    // N = 14336 16.7 against 20.2 us with waves that split K)
+    // N = 14336 16.7 against 20.2 us with waves that split K -- as long as all workgroups are resident at once: with
+    // N = 28672 and two rounds of them 31.6 against 26.2)
+    size_t max_row_bytes = row ? 32 * 1024 : 16 * 1024;
+    if (row && m > 4 && a_bytes <= kMaxLdsBytes &&
+        (tiles + 3) / 4 <= kComputeUnits * static_cast<int>(kMaxLdsBytes / a_bytes)) {
+      max_row_bytes = kMaxLdsBytes;
+    }
     const bool rings_fit_k =
         5 * requested_slices(k, 16, 2) < 6 * slices || 5 * requested_slices(k, 8, 4) < 6 * slices;
     const int min_tiles = row ? 896 : rings_fit_k ? 2000 : 832;
@@ -399,6 +407,11 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
     const int col_groups = (tiles + nt - 1) / nt;
     if (!row && col_groups > kComputeUnits && 20 * requested_slices(k, 8, d8) <= 21 * requested_slices(k, 16, 2)) {
       set(d8, nt, 1, 8, kRowsWholeInLds, 8);
+    } else if (row && m > 4 && k <= 8192) {
+      // blocks along N, five to sixteen rows: eight waves with four slices in flight and the rows staged per slice
+      // (measured against the sixteen-wave shape: M = 16, K = N = 4096 6.6 against 7.2 us, M = 8, N = 11008 15.8
+      // against 16.9)
+      set(4, 1, 1, 8, kRowsPerSlotInLds, 8);
     } else {
       set(2, nt, 1, 16, kRowsWholeInLds, 16);
     }
@@ -607,8 +620,8 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
     const double streaming_us = 3.2 + static_cast<double>(rounds) * (0.44 + s.nt * (0.69 + 0.37 * (static_cast<double>(k) / 1024.0)));
     return streaming_us < tile_us;
   }
-  if (m <= 32) return true;
-  // more row groups, and blocks along N, where the streaming kernel converts with 23 instead of 13 instructions per 8
+  // more row groups, and blocks along N (from 17 rows on: M = 32, K = 8192, N = 28672 with blocks along N takes 80 us
+  // streaming and 50 in 64 x 128 tiles), where the streaming kernel converts with 23 instead of 13 instructions per 8
   // weights
   double streaming_us = (column_wise ? 2.8 : 5.6) * static_cast<double>(row_groups) * (static_cast<double>(n) / 4096.0) *
                         (static_cast<double>(k) / 4096.0);

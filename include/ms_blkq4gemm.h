@@ -269,6 +269,38 @@ int blkq4_gemm_plan_sm80(
     void* error_message);
 
 /**
+ * blkq4_fp16_gemm_sm80 / blkq4_bf16_gemm_sm80 (bf16 != 0) with the kernel given by the caller instead of the library's
+ * cost model.  `plan` is text:
+ *   "auto"                                     what the cost model picks (then identical to the entry points above);
+ *   "tile RT NT WM WN PW KW PARTS"             the tile kernel: WM x WN computing waves of (32 RT) x (32 NT) outputs, PW
+ *                                              producer waves, KW = 4 for the tiles whose waves split the k tile (else
+ *                                              1), the tiles of the last round shared out over PARTS workgroups along K;
+ *   "streaming DEPTH NT MT WAVES ROWS SPLIT"   the weight-streaming kernel: slices in flight, column tiles and row tiles
+ *                                              (1: up to 16 rows, 2: row groups of 32) per workgroup, waves, rows whole
+ *                                              in LDS (1) or staged per slice (2), SPLIT = WAVES or 1;
+ *   "decode ROWS NT WAVES DEPTH"               the decode kernel: rows kept, column tiles per workgroup, waves, slices each.
+ * The shapes that exist are the ones blkq4_gemm_plan_sm80 can name; any other, or one that does not fit the problem, is
+ * refused with -1 before anything is launched.  Same arguments, checks and results (to the stated tolerance; the
+ * reference's exact construction stays exact) as the entry points above.
+ *
+ * No counterpart in the reference, whose choice is a single `m > 16` (src/blkq4_f16_gemm_sm80.cu:343): it exists so
+ * that the cost model's choices can be measured against the alternatives on a given machine (bench.py --check-plans).
+ */
+int blkq4_gemm_with_plan_sm80(
+  const char* plan,
+  int block_size,
+  bool column_wise_blocking,
+  bool bf16,
+  int m, int n, int k,
+  void* stream,
+  void const* act_ptr, size_t a_size,
+  void const* weights_ptr, size_t weights_size,
+  void const* scales_ptr, size_t scales_size,
+  void const* offsets_ptr, size_t offsets_size,
+  void* output_ptr, size_t output_size,
+  void* error_message);
+
+/**
  * The workspaces of the GEMM's split plans (see "Device memory and state" at the top).  Host-side bookkeeping; no
  * kernel is launched.
  *   blkq4_gemm_workspace_info_sm80: *state = 1 when a GEMM issued on `stream` now (in the recording the stream is

@@ -172,3 +172,32 @@ def test_repack_validation_messages(capi):
 def test_error_message_may_be_null(capi):
     lib = capi.load()
     assert lib.blkq4_fp16_gemm_sm80(32, True, 0, 64, 64, None, None, 0, None, 0, None, 0, None, 0, None, 0, None) == -1
+
+
+@pytest.mark.parametrize("plan,message", [
+    ("spiral 3", "Unknown plan: a plan is"),
+    ("tile 4 2 1 4", "Unknown plan: a plan is"),
+    ("tile 0 2 1 4 4 1 1", "Unknown plan: tile RT NT WM WN PW KW PARTS"),
+    ("streaming 2 1 3 8 1 8", "Unknown plan: streaming DEPTH NT MT WAVES ROWS SPLIT"),
+    ("streaming 2 1 1 8 1 4", "Unknown plan: streaming DEPTH NT MT WAVES ROWS SPLIT"),
+    ("decode 32 1 8 4", "Unknown plan: decode ROWS NT WAVES DEPTH"),
+    # plans that parse but name no kernel, or a kernel that does not fit the problem: refused by the launchers,
+    # before anything is launched
+    ("tile 3 3 1 4 4 1 1", "Kernel execution failed: invalid argument"),
+    ("tile 4 1 1 1 4 2 1", "Kernel execution failed: invalid argument"),
+    ("streaming 3 1 1 8 1 8", "Kernel execution failed: invalid argument"),
+    ("decode 1 1 8 4", "Kernel execution failed: invalid argument"),     # 4 rows do not fit a kernel that keeps 1
+    ("decode 4 1 8 4", "Kernel execution failed: invalid argument"),     # K = 512 is 4 slices, not 32
+])
+def test_plans_given_as_text_are_checked(capi, plan, message):
+    """blkq4_gemm_with_plan_sm80: what is no plan is refused by the parser, what is no kernel by the launchers."""
+    m, n, k, bs = 4, 64, 512, 32
+    with pytest.raises(capi.Blkq4Error) as e:
+        capi.gemm_with_plan(plan, bs, True, m, n, k, _buf(m * k * 2), _buf(k * n // 2), _buf((k // bs) * n * 2), None,
+                            _buf(m * n * 2), stream=0)
+    assert str(e.value).startswith(message), str(e.value)
+
+
+def test_plan_entry_point_validates_like_the_gemm(capi):
+    with pytest.raises(capi.Blkq4Error, match="Unexpected activation tensor size: 10 expected: 4096"):
+        capi.gemm_with_plan("auto", 32, True, 4, 64, 512, _buf(10), _buf(512 * 32), _buf(16 * 64 * 2), None, _buf(512), stream=0)
