@@ -366,10 +366,22 @@ def bench_prepack(torch, capi, device, steps, warmup, with_cpu=True):
     wall, evt, mode = timed_region(torch, launches, steps, max(2, warmup // 10))
     per = evt / steps
     ach = nbytes / per / 1e9
+    # the same bytes moved the same way with no arithmetic (the probe library's twin of the kernel), same run
+    import ctypes
+    import bench_probe
+    probe = ctypes.CDLL(bench_probe.build())
+    vp = ctypes.c_void_p
+    probe.blkq4_probe_prepack_traffic.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp, vp]
+    t_w, t_s, t_z = torch.empty_like(q_w), torch.empty_like(q_s), torch.empty_like(q_zp)
+    twin = [lambda: probe.blkq4_probe_prepack_traffic(w.data_ptr(), k, n, k, t_w.data_ptr(), t_s.data_ptr(), t_z.data_ptr(),
+                                                     vp(torch.cuda.current_stream().cuda_stream))]
+    _, twin_evt, _ = timed_region(torch, twin, steps, max(2, warmup // 10))
+    del t_w, t_s, t_z
     res = {
         "workload": "C5 quantize+prepack K=8192 N=28672 bs16 asym", "value": round(nbytes / (wall / steps) / 1e9, 3),
         "unit": "GB/s", "ms_per_step": round(wall / steps * 1e3, 6), "kernel_us": round(per * 1e6, 3), "timing": mode,
         "launches_per_region": steps, "bytes": nbytes, "gbps": round(ach, 3),
+        "traffic_only_twin_us": round(twin_evt / steps * 1e6, 3),
         "roofline": {"bound": "hbm", "achieved": round(ach, 3), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                      "frac": round(ach / PEAK_HBM_GBPS, 4), "traffic": traffic_bytes("C5_prepack")},
     }
@@ -498,7 +510,7 @@ def bench_context(torch, capi, device, head_problem, steps, warmup):
                     for w, sc in zip(ws, ss)]
         wall, evt, _ = timed_region(torch, launches, floor_launches, warmup)
         out["c2_requests_only_us" if with_scales else "c2_weight_requests_only_us"] = round(evt / floor_launches * 1e6, 3)
-    # the same bytes requested the way the decode kernel requests them (four waves, eight slices each, at once)
+    # the same bytes requested the way the decode kernel requests them (eight waves, four slices each, at once)
     probe.blkq4_probe_decode_requests.argtypes = probe.blkq4_probe_stream.argtypes
     launches = [(lambda w=w, sc=sc: probe.blkq4_probe_decode_requests(w.data_ptr(), sc.data_ptr(), n, k, scratch.data_ptr(), stream_ptr()))
                 for w, sc in zip(ws, ss)]
@@ -609,6 +621,8 @@ def main(argv=None) -> int:
         r = res.get("roofline")
         if r is not None and key != "copy":
             by_workload[key] = {"bound": r["bound"], "frac": r["frac"], "kernel_us": res["kernel_us"]}
+            if "traffic_only_twin_us" in res:
+                by_workload[key]["traffic_only_twin_us"] = res["traffic_only_twin_us"]
     line["roofline"]["by_workload"] = by_workload
     if "C2" in results:
         c2 = results["C2"]

@@ -61,6 +61,61 @@ __global__ __launch_bounds__(64 * WAVES) void decode_requests_kernel(const uint8
   if (a == 0x12345678u) out[blockIdx.x] = a;  // keeps the loads alive, (almost) never stores
 }
 
+// The quantizer's memory traffic and nothing else: the tile, the loads, the trip through LDS and the stores of the
+// product's kernel for blocks of BS along K with zero-points (32 columns x 256 rows per workgroup, four 16-byte
+// non-temporal loads per lane, packed words 16 bytes per lane, scales 8 and zero-points 4 bytes per lane), with an
+// exclusive-or in place of the arithmetic.  What it takes is what the quantizer cannot go below without moving
+// its bytes differently.
+typedef unsigned probe_u32x4 __attribute__((ext_vector_type(4)));
+template <int BS>
+__global__ __launch_bounds__(256) void prepack_traffic_kernel(const uint16_t* __restrict__ src, int K, int N, int ld,
+                                                             uint4* __restrict__ packed_w, uint16_t* __restrict__ scales,
+                                                             uint8_t* __restrict__ zps, unsigned k_tiles) {
+  constexpr int kTileN = 32, kTileK = 256, kBlocksPerTile = kTileK / BS;
+  __shared__ uint32_t w_lds[kTileK / 32][kTileN][4];
+  __shared__ __attribute__((aligned(8))) uint16_t s_lds[kBlocksPerTile][kTileN];
+  __shared__ __attribute__((aligned(4))) uint8_t z_lds[kBlocksPerTile][kTileN];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int k0 = static_cast<int>(blockIdx.x % k_tiles) * kTileK, n0 = static_cast<int>(blockIdx.x / k_tiles) * kTileN;
+  const int kl = (lane & 31) * 8;
+  probe_u32x4 raw[4];
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int nl = wave * 8 + it * 2 + (lane >> 5);
+    raw[it] = __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4*>(
+        src + static_cast<size_t>(min(n0 + nl, N - 1)) * ld + min(k0 + kl, K - 8)));
+  }
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int nl = wave * 8 + it * 2 + (lane >> 5);
+    const uint32_t word = raw[it][0] ^ raw[it][1] ^ raw[it][2] ^ raw[it][3];
+    w_lds[kl >> 5][nl][(kl >> 3) & 3] = word;
+    if ((kl % BS) == 0) {
+      s_lds[kl / BS][nl] = static_cast<uint16_t>(word);
+      z_lds[kl / BS][nl] = static_cast<uint8_t>(word >> 16);
+    }
+  }
+  __syncthreads();
+  {
+    const int ksl = tid / kTileN, nl = tid % kTileN;
+    const int k = k0 + ksl * 32, n = n0 + nl;
+    if (k < K && n < N) {
+      const uint4 v = *reinterpret_cast<const uint4*>(&w_lds[ksl][nl][0]);
+      __builtin_nontemporal_store(probe_u32x4{v.x, v.y, v.z, v.w},
+                                  reinterpret_cast<probe_u32x4*>(&packed_w[static_cast<size_t>(k >> 5) * N + n]));
+    }
+  }
+  for (int u = tid; u < kBlocksPerTile * kTileN / 4; u += 256) {
+    const int bl = u / (kTileN / 4), nl = (u % (kTileN / 4)) * 4;
+    const int k = k0 + bl * BS, n = n0 + nl;
+    if (k < K && n < N) {
+      const size_t idx = static_cast<size_t>(k / BS) * N + n;
+      *reinterpret_cast<uint2*>(scales + idx) = *reinterpret_cast<const uint2*>(&s_lds[bl][nl]);
+      *reinterpret_cast<uint32_t*>(zps + idx) = *reinterpret_cast<const uint32_t*>(&z_lds[bl][nl]);
+    }
+  }
+}
+
 typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
 typedef float probe_float16 __attribute__((ext_vector_type(16)));
 
@@ -151,11 +206,11 @@ PROBE_EXPORT int blkq4_probe_stream16(const void* packed_w, const void* scales, 
   return static_cast<int>(hipGetLastError());
 }
 
-// the decode kernel's requests: four waves with eight slices each (k = 4096)
+// the decode kernel's requests: eight waves with four slices each (k = 4096)
 PROBE_EXPORT int blkq4_probe_decode_requests(const void* packed_w, const void* scales, int n, int k, void* scratch,
                                              void* stream) {
   if (n % 16 != 0 || k != 4096) return static_cast<int>(hipErrorInvalidValue);
-  hipLaunchKernelGGL((decode_requests_kernel<4, 8>), dim3(n / 16), dim3(256), 0, static_cast<hipStream_t>(stream),
+  hipLaunchKernelGGL((decode_requests_kernel<8, 4>), dim3(n / 16), dim3(512), 0, static_cast<hipStream_t>(stream),
                      static_cast<const uint8_t*>(packed_w), static_cast<const uint8_t*>(scales),
                      static_cast<unsigned*>(scratch), n);
   return static_cast<int>(hipGetLastError());
@@ -171,5 +226,17 @@ PROBE_EXPORT int blkq4_probe_mfma(int random_operands, int iters, void* scratch,
     hipLaunchKernelGGL(mfma_kernel<false>, dim3(256), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<float*>(scratch), iters);
   }
+  return static_cast<int>(hipGetLastError());
+}
+
+// src: fp16 [n][ld]; packed_w k n / 2 bytes, scales (k / 16) n fp16 (8-byte aligned), zps (k / 16) n bytes (4-byte
+// aligned): the buffers of the quantizer for blocks of 16 along K; k a multiple of 64, n of 32
+PROBE_EXPORT int blkq4_probe_prepack_traffic(const void* src, int k, int n, int ld, void* packed_w, void* scales, void* zps,
+                                             void* stream) {
+  if (k % 64 != 0 || n % 32 != 0) return static_cast<int>(hipErrorInvalidValue);
+  const unsigned k_tiles = (k + 255) / 256;
+  hipLaunchKernelGGL(prepack_traffic_kernel<16>, dim3(k_tiles * (n / 32)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(src), k, n, ld, static_cast<uint4*>(packed_w),
+                     static_cast<uint16_t*>(scales), static_cast<uint8_t*>(zps), k_tiles);
   return static_cast<int>(hipGetLastError());
 }

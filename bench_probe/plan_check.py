@@ -30,6 +30,8 @@ VARIANTS = {
     "fp16/bs32/sym": (False, 32, True, False),
     "fp16/bs64/along-N": (False, 64, False, True),
 }
+# the variant the constants were fitted on, for --shapes
+FITTED_VARIANTS = {"fp16/bs64": (False, 64, True, True), "fp16/bs64/sym": (False, 64, True, False)}
 LAYERS = [(4096, 4096), (11008, 4096), (4096, 11008), (28672, 8192), (14336, 4096)]   # (N, K)
 ROWS = [1, 4, 8, 16, 32, 64, 128, 256, 512]
 
@@ -120,7 +122,7 @@ def time_plan(torch, launch_on_set, sets, settle, regions=3):
 
 
 def check_shape(torch, capi, device, variant, m, n, k, settle):
-    bf16, bs, column_wise, has_zp = VARIANTS[variant]
+    bf16, bs, column_wise, has_zp = {**VARIANTS, **FITTED_VARIANTS}[variant]
     dtype = torch.bfloat16 if bf16 else torch.float16
     per_set = k * n // 2 + 2 * k * n // bs + (k * n // bs if has_zp else 0)
     streams_weights = m <= 128

@@ -119,9 +119,10 @@ inline bool streaming_takes_few_rows(int m, int n, int k) {
 //
 // Waves.  Eight by default (measured on M = 1, rotating weights, against 4 and 16 waves: K = 2048, N = 2048: 2.62
 // against 2.74 and 2.68 us; K = 4096, N = 11008: 6.54 against 6.64 and 7.06; N = 128256: 49.1 against 50.2 and 58.3;
-// K = 8192, N = 4096: 5.41 against 16 waves' 5.40), four for short K, and for one workgroup per compute unit at most
-// when they then request eight slices each (K = 4096, N = 4096: 3.68 against 3.74 and 3.80 us), sixteen when eight
-// would have to request more than eight slices each (up to four rows only).
+// K = 8192, N = 4096: 5.41 against 16 waves' 5.40), four for short K, sixteen when eight would have to request more
+// than eight slices each (up to four rows only).  (Four waves with eight slices each for one workgroup per compute
+// unit, K = N = 4096, were the rule once: without zero-points the two are level, 3.71 against 3.70 us; with zero-points
+// eight waves take 3.70 against 3.86, in bf16 3.91 against 4.07.)
 //
 // Column tiles per workgroup.  The busiest compute unit works through ceil(workgroups / 256) workgroups of nt
 // tiles each, and every workgroup costs a fraction of a tile's work on top: staging the rows, the instructions
@@ -162,7 +163,7 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
   const int rows = m == 1 ? 1 : m <= 4 ? 4 : m <= 8 ? 8 : 16;
   int waves = 8;
   if (rows <= 4) {
-    if (slices <= 8 || (slices > 24 && slices <= 32 && tiles <= kComputeUnits)) waves = 4;
+    if (slices <= 8) waves = 4;
     if (slices > 8 * kDecodeMaxDepth) waves = 16;
     if (slices > 16 * kDecodeMaxDepthSixteenWaves) return false;
   }

@@ -46,7 +46,7 @@ def test_benchmark_configurations_get_the_expected_families(capi):
     plans = {name: capi.gemm_plan(bs, True, m, n, k, has_offsets=zp)[2] for name, (m, k, n, bs, zp) in {
         "C1": (64, 1024, 1024, 32, True), "C2": (1, 4096, 4096, 64, False), "C3": (16, 4096, 11008, 32, True),
         "C4": (2048, 4096, 4096, 64, True), "C5": (4096, 8192, 28672, 16, True)}.items()}
-    assert plans["C2"] == "decode: 4 waves splitting K, 8 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups"
+    assert plans["C2"] == "decode: 8 waves splitting K, 4 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups"
     assert plans["C3"] == "decode: 8 waves splitting K, 4 slices requested by each, 3 column tile(s) x 16 row(s), 230 workgroups"
     assert plans["C1"].startswith("streaming:")
     assert plans["C4"].startswith("tile: 128 x 256, 4 + 4 waves, 256 tiles") and "parts" not in plans["C4"]
