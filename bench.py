@@ -87,29 +87,29 @@ DESCRIPTION = {
 # figure of a workload is reported only while the library still picks the kernel it was taken from (TRAFFIC_KERNEL).
 COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65552.0, "WRITE_SIZE": 1.0}
 COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
-    "C4": (44138.2, 16386.4),
-    "C2": (4429.6, 8.0),
-    "C3": (13653.6, 344.0),
-    "C5": (860409.6, 229384.7),
-    "C5_prepack": (229443.7, 157730.3),
-    "C4r": (44141.6, 16386.0),
+    "C4": (44132.6, 16387.0),
+    "C2": (4406.1, 8.0),
+    "C3": (13653.7, 344.0),
+    "C5": (860380.2, 229382.3),
+    "C5_prepack": (229410.8, 157706.9),
+    "C4r": (44141.1, 16385.9),
     "C2r": (4428.1, 8.0),
-    "C1": (869.5, 128.0),
-    "M128": (8650.6, 1024.0),
-    "M256": (24163.1, 11216.5),
-    "M512": (37966.5, 4266.3),
-    "M768N11K": (60858.5, 16514.9),
-    "M256K11K": (43371.1, 19433.4),
-    "V128K": (136348.9, 251.0),
-    "B16": (64098.7, 896.0),
-    "C4b": (44167.5, 16387.6),
-    "C2b": (4441.1, 8.0),
+    "C1": (869.0, 128.0),
+    "M128": (8649.1, 1024.0),
+    "M256": (14387.1, 2048.0),
+    "M512": (37967.6, 4270.0),
+    "M768N11K": (60863.0, 16513.7),
+    "M256K11K": (43374.1, 19434.3),
+    "V128K": (136348.8, 250.8),
+    "B16": (64097.7, 896.0),
+    "C4b": (44164.5, 16387.0),
+    "C2b": (4418.6, 8.0),
 }
 
 
 TRAFFIC_KERNEL = {  # what blkq4_gemm_plan_sm80 said the workload runs when its counters were taken
     "C1": "streaming: 8 waves splitting K, 1 column tile(s) x 32 rows, 2 slices in flight, rows whole in LDS, 2 row group(s), 128 workgroups",
-    "C2": "decode: 4 waves splitting K, 8 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
+    "C2": "decode: 8 waves splitting K, 4 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
     "C3": "decode: 8 waves splitting K, 4 slices requested by each, 3 column tile(s) x 16 row(s), 230 workgroups",
     "C4": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
     "C5": "tile: 256 x 256, 4 + 0 waves, 1792 tiles",
@@ -119,8 +119,8 @@ TRAFFIC_KERNEL = {  # what blkq4_gemm_plan_sm80 said the workload runs when its 
     "V128K": "decode: 8 waves splitting K, 4 slices requested by each, 2 column tile(s) x 1 row(s), 4008 workgroups",
     "B16": "streaming: 8 waves splitting K, 7 column tile(s) x 16 rows, 2 slices in flight, rows staged per slice, 1 row group(s), 256 workgroups",
     "C4b": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
-    "C2b": "decode: 4 waves splitting K, 8 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
-    "M256": "tile: 64 x 128, 4 + 4 waves, 128 tiles, the last 128 in 2 parts (workspace 8404992 bytes)",
+    "C2b": "decode: 8 waves splitting K, 4 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
+    "M256": "tile: 128 x 32, 4 + 4 waves (the computing waves split the k tile), 256 tiles",
     "M512": "tile: 64 x 128, 4 + 4 waves, 256 tiles",
     "M768N11K": "tile: 256 x 256, 4 + 0 waves, 129 tiles",
     "M256K11K": "tile: 128 x 128, 4 + 4 waves, 64 tiles, the last 64 in 4 parts (workspace 16793600 bytes)",
