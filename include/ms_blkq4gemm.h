@@ -284,7 +284,7 @@ int blkq4_gemm_plan_sm80(
  * reference's exact construction stays exact) as the entry points above.
  *
  * No counterpart in the reference, whose choice is a single `m > 16` (src/blkq4_f16_gemm_sm80.cu:343): it exists so
- * that the cost model's choices can be measured against the alternatives on a given machine (bench.py --check-plans).
+ * that the cost model's choices can be measured against the alternatives on a given machine (`python -m bench_probe.plan_check`).
  */
 int blkq4_gemm_with_plan_sm80(
   const char* plan,
