@@ -290,3 +290,28 @@ def test_non_default_stream(oracle, capi, device):
         capi.gemm(64, True, 8, 256, 256, a_dev, q_w, q_s, q_zp, out, stream=s)
     s.synchronize()
     assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("m,n,k,plans", [
+    (16, 1024, 1024, ["auto", "decode 16 1 8 1", "decode 16 2 8 1", "streaming 4 1 1 8 1 8", "streaming 2 1 1 16 1 16"]),
+    (200, 2048, 2048, ["auto", "tile 2 1 1 4 4 1 1", "tile 4 1 1 4 4 1 1", "tile 4 1 1 4 4 1 2", "tile 4 2 1 4 4 1 1",
+                       "tile 8 2 1 4 0 1 1", "tile 8 1 1 4 4 1 1", "tile 4 1 1 1 4 4 1", "streaming 2 4 2 8 1 8",
+                       "streaming 2 2 2 8 2 8"]),
+])
+def test_every_plan_given_as_text_is_exact_on_reference_construction(oracle, capi, device, m, n, k, plans):
+    """blkq4_gemm_with_plan_sm80: whichever kernel is asked for by name, the reference's exact construction
+    (test/blkq4_fp16_gemm_sm80_test.cu:194-256,469-472) comes out bit for bit."""
+    bs, has_offsets = 64, True
+    rng = np.random.default_rng(m + n + k)
+    kat = oracle.kat_generate(bs, True, k, n, has_offsets)
+    a = grid_activations(rng, m, k)
+    q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, kat["weights"], has_offsets)
+    ref = oracle.gemm(a, kat["weights"])
+    a_dev = to_dev(a, device)
+    for plan in plans:
+        out = torch.full((m, n), float("nan"), dtype=torch.float16, device=device)
+        capi.gemm_with_plan(plan, bs, True, m, n, k, a_dev, q_w, q_s, q_zp, out)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16)), plan
+    with pytest.raises(capi.Blkq4Error, match="Kernel execution failed: invalid argument"):
+        capi.gemm_with_plan("decode 16 1 8 2", bs, True, m, n, k, a_dev, q_w, q_s, q_zp, out)   # K is not 16 slices
