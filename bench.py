@@ -97,7 +97,7 @@ COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
     "C1": (869.0, 128.0),
     "M128": (8649.1, 1024.0),
     "M256": (14387.1, 2048.0),
-    "M512": (37967.6, 4270.0),
+    "M512": (17233.5, 4183.2),
     "M768N11K": (60863.0, 16513.7),
     "M256K11K": (43374.1, 19434.3),
     "V128K": (136348.8, 250.8),
@@ -121,7 +121,7 @@ TRAFFIC_KERNEL = {  # what blkq4_gemm_plan_sm80 said the workload runs when its 
     "C4b": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
     "C2b": "decode: 8 waves splitting K, 4 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
     "M256": "tile: 128 x 32, 4 + 4 waves (the computing waves split the k tile), 256 tiles",
-    "M512": "tile: 64 x 128, 4 + 4 waves, 256 tiles",
+    "M512": "tile: 64 x 128, 4 + 4 waves, 256 tiles, blocks of 4 x 8 tiles per XCD",
     "M768N11K": "tile: 256 x 256, 4 + 0 waves, 129 tiles",
     "M256K11K": "tile: 128 x 128, 4 + 4 waves, 64 tiles, the last 64 in 4 parts (workspace 16793600 bytes)",
 }

@@ -155,6 +155,47 @@ __global__ __launch_bounds__(256) void mfma_kernel(float* out, int iters) {
   out[blockIdx.x * blockDim.x + threadIdx.x] = sum;
 }
 
+
+// What a wave's own instruction stream costs: `iters` rounds of four independent MFMAs (32 x 32 x 16, fp16), each
+// followed by N independent packed vector instructions.  Every wave leaves its cycle count (s_memtime) per MFMA in
+// cycles[wave]; with one workgroup the waves' figures show how waves of one SIMD share it.
+typedef _Float16 probe_half8_t __attribute__((ext_vector_type(8)));
+typedef float probe_float16_t __attribute__((ext_vector_type(16)));
+template <int N>
+__global__ __launch_bounds__(1024) void issue_kernel(unsigned long long* cycles, int iters, unsigned seed) {
+  probe_half8_t a, b;
+  for (int e = 0; e < 8; ++e) {
+    a[e] = static_cast<_Float16>(static_cast<float>((threadIdx.x + e + seed) & 7));
+    b[e] = static_cast<_Float16>(static_cast<float>((e * 3 + seed) & 7));
+  }
+  probe_float16_t acc[4];
+  for (int g = 0; g < 4; ++g)
+    for (int e = 0; e < 16; ++e) acc[g][e] = 0.f;
+  unsigned x[8];
+  for (int j = 0; j < 8; ++j) x[j] = seed + j + threadIdx.x;
+  const unsigned c = seed * 3 + 1;
+  const unsigned long long t0 = __builtin_amdgcn_s_memtime();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      acc[g] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[g], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < N; ++j) asm volatile("v_pk_add_f16 %0, %0, %1" : "+v"(x[(g * N + j) % 8]) : "v"(c));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memtime();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  float s = 0;
+  for (int g = 0; g < 4; ++g)
+    for (int e = 0; e < 16; ++e) s += acc[g][e];
+  unsigned y = 0;
+  for (int j = 0; j < 8; ++j) y ^= x[j];
+  if ((threadIdx.x & 63) == 0 && blockIdx.x == 0) cycles[threadIdx.x >> 6] = (t1 - t0) / (4ull * iters);
+  if (s == 12345.678f && y == 77) cycles[63] = 1;  // keeps the work alive, (almost) never stores
+}
+
 }  // namespace
 
 #define PROBE_EXPORT extern "C" __attribute__((visibility("default")))
@@ -238,5 +279,24 @@ PROBE_EXPORT int blkq4_probe_prepack_traffic(const void* src, int k, int n, int 
   hipLaunchKernelGGL(prepack_traffic_kernel<16>, dim3(k_tiles * (n / 32)), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const uint16_t*>(src), k, n, ld, static_cast<uint4*>(packed_w),
                      static_cast<uint16_t*>(scales), static_cast<uint8_t*>(zps), k_tiles);
+  return static_cast<int>(hipGetLastError());
+}
+
+// `workgroups` workgroups of `threads` threads (64 ... 1024), 4 * iters MFMAs per wave, each followed by
+// vector_per_mfma (0, 2, 4, 6, 8, 12 or 16) independent vector instructions; cycles: 64 x 8 bytes of device memory
+// that receive workgroup 0's cycles per MFMA, wave by wave.  Flop of the launch: workgroups * threads / 64 * iters * 4 * 32768.
+PROBE_EXPORT int blkq4_probe_issue(int vector_per_mfma, int workgroups, int threads, int iters, void* cycles, void* stream) {
+  if (threads < 64 || threads > 1024 || threads % 64 != 0 || workgroups < 1 || iters < 1) return static_cast<int>(hipErrorInvalidValue);
+#define PROBE_ISSUE_CASE(N_)                                                                                          \
+  case N_:                                                                                                            \
+    hipLaunchKernelGGL(issue_kernel<N_>, dim3(workgroups), dim3(threads), 0, static_cast<hipStream_t>(stream),        \
+                       static_cast<unsigned long long*>(cycles), iters, 1u);                                          \
+    break;
+  switch (vector_per_mfma) {
+    PROBE_ISSUE_CASE(0) PROBE_ISSUE_CASE(2) PROBE_ISSUE_CASE(4) PROBE_ISSUE_CASE(6) PROBE_ISSUE_CASE(8) PROBE_ISSUE_CASE(12)
+    PROBE_ISSUE_CASE(16)
+    default: return static_cast<int>(hipErrorInvalidValue);
+  }
+#undef PROBE_ISSUE_CASE
   return static_cast<int>(hipGetLastError());
 }

@@ -2,7 +2,7 @@
 plan ``blkq4_gemm_plan_sm80`` names ("auto") and with every other plan that exists for it, forced through
 ``blkq4_gemm_with_plan_sm80``; one JSON line per shape says what was chosen, what was fastest and by how much.
 
-    python -m bench_probe.plan_check [--part i/n] [--quick]
+    python -m bench_probe.plan_check [--part i/n] [--quick] [--shapes variant:m:n:k,...] [--every-plan]
 
 The shapes cover what the constants of the model were NOT fitted on: bf16, blocks of 16 and 32, blocks along N, next to
 M = 1 ... 512, N = 4096 ... 28672, K = 4096 ... 11008.  Weight sets rotate over more than the Infinity Cache for the
@@ -67,6 +67,11 @@ def candidate_plans(column_wise, m, n, k):
                 if parts > 1 and (kw > 1 or rt == 1 or (rt == 2 and wn == 8) or rem * parts > 256 or kt // parts < 4):
                     continue
                 plans.append(f"tile {rt} {nt} {wm} {wn} {pw} {kw} {parts}")
+                # the tile order of whole rounds dealt to the XCDs in blocks (1, 2, 4 or 8 row bands)
+                m_tiles = -(-m // (32 * rt * wm))
+                if parts == 1 and tiles >= 256 and m_tiles & (m_tiles - 1) == 0:
+                    plans += [f"tile {rt} {nt} {wm} {wn} {pw} {kw} 1 {bands}" for bands in (1, 2, 4, 8)
+                              if bands <= m_tiles <= 32 * bands]
     if m <= 16:
         plans += ["streaming 2 1 1 16 1 16", "streaming 2 2 1 16 1 16", "streaming 4 1 1 8 1 8", "streaming 4 2 1 8 1 8",
                   "streaming 4 1 1 4 1 1", "streaming 2 4 1 8 2 8", "streaming 2 4 1 4 2 4", "streaming 2 7 1 8 2 8",
@@ -121,7 +126,7 @@ def time_plan(torch, launch_on_set, sets, settle, regions=3):
     return times[len(times) // 2]
 
 
-def check_shape(torch, capi, device, variant, m, n, k, settle):
+def check_shape(torch, capi, device, variant, m, n, k, settle, every_plan=False):
     bf16, bs, column_wise, has_zp = {**VARIANTS, **FITTED_VARIANTS}[variant]
     dtype = torch.bfloat16 if bf16 else torch.float16
     per_set = k * n // 2 + 2 * k * n // bs + (k * n // bs if has_zp else 0)
@@ -167,10 +172,13 @@ def check_shape(torch, capi, device, variant, m, n, k, settle):
     chosen_us = timed["auto"]
     forced = {p: t for p, t in timed.items() if p != "auto"}
     best_plan = min(forced, key=forced.get)
-    return {"variant": variant, "m": m, "n": n, "k": k, "weight_sets": copies, "chosen": chosen_text, "chosen_us": chosen_us,
-            "best_forced": best_plan, "best_forced_us": forced[best_plan],
-            "chosen_over_best": round(chosen_us / min(chosen_us, forced[best_plan]), 3),
-            "wrong_results": [p for p, r in results.items() if "error" in r], "plans_timed": len(timed)}
+    row = {"variant": variant, "m": m, "n": n, "k": k, "weight_sets": copies, "chosen": chosen_text, "chosen_us": chosen_us,
+           "best_forced": best_plan, "best_forced_us": forced[best_plan],
+           "chosen_over_best": round(chosen_us / min(chosen_us, forced[best_plan]), 3),
+           "wrong_results": [p for p, r in results.items() if "error" in r], "plans_timed": len(timed)}
+    if every_plan:
+        row["us_by_plan"] = forced
+    return row
 
 
 def main(argv=None) -> int:
@@ -178,6 +186,7 @@ def main(argv=None) -> int:
     ap.add_argument("--part", default="1/1", help="i/n: the i-th of n slices of the shape list")
     ap.add_argument("--quick", action="store_true", help="shorter settle phase")
     ap.add_argument("--shapes", default="", help="variant:m:n:k,... instead of the built-in list")
+    ap.add_argument("--every-plan", action="store_true", help="print every forced plan's time, not only the best one's")
     args = ap.parse_args(argv)
     import torch
     from gemmlib_amd import capi
@@ -190,7 +199,7 @@ def main(argv=None) -> int:
         todo = [(v, int(m), int(n), int(k)) for v, m, n, k in (item.split(":") for item in args.shapes.split(","))]
     rows = []
     for variant, m, n, k in todo:
-        row = check_shape(torch, capi, device, variant, m, n, k, 0.05 if args.quick else 0.15)
+        row = check_shape(torch, capi, device, variant, m, n, k, 0.05 if args.quick else 0.15, args.every_plan)
         rows.append(row)
         print(json.dumps(row), flush=True)
         torch.cuda.empty_cache()

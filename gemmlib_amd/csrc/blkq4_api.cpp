@@ -204,17 +204,19 @@ int launch_choice(const blkq4::Choice& choice, bool bf16, const blkq4_gemm_args*
 bool parse_plan(const char* text, bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity,
                 blkq4::Choice* c, std::string* why) {
   *c = blkq4::Choice{};
-  int v[7] = {0, 0, 0, 0, 0, 0, 0};
+  int v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   if (text == nullptr || std::strcmp(text, "auto") == 0) {
     *c = blkq4::choose(column_wise, bf16, m, n, k, workspace_capacity);
     return true;
   }
-  if (std::sscanf(text, "tile %d %d %d %d %d %d %d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5], &v[6]) == 7) {
+  if (std::sscanf(text, "tile %d %d %d %d %d %d %d %d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5], &v[6], &v[7]) >= 7) {
     auto& t = c->t;
     c->family = blkq4::kFamilyTile;
     t.rt = v[0]; t.nt = v[1]; t.wm = v[2]; t.wn = v[3]; t.pw = v[4]; t.kw = v[5];
-    if (t.rt < 1 || t.nt < 1 || t.wm < 1 || t.wn < 1 || t.pw < 0 || t.kw < 1 || v[6] < 1 || t.rt * t.wm > 64 || t.nt * t.wn > 64) {
-      *why = "tile RT NT WM WN PW KW PARTS: positive numbers (PW may be 0, PARTS 1 means no split)";
+    t.xcd_rows = v[7];
+    if (t.rt < 1 || t.nt < 1 || t.wm < 1 || t.wn < 1 || t.pw < 0 || t.kw < 1 || v[6] < 1 || v[7] < 0 || t.rt * t.wm > 64 || t.nt * t.wn > 64) {
+      *why = "tile RT NT WM WN PW KW PARTS [BANDS]: positive numbers (PW may be 0, PARTS 1 means no split, BANDS 0 or absent: "
+             "tile order as it is)";
       return false;
     }
     t.tiles = static_cast<int>(blkq4::ceil_div(m, 32 * t.rt * t.wm) * blkq4::ceil_div(n, 32 * t.nt * t.wn));
@@ -265,7 +267,7 @@ bool parse_plan(const char* text, bool column_wise, bool bf16, int m, int n, int
     d.lds_bytes = static_cast<uint32_t>(blkq4::decode_lds_bytes(d.row != 0, d.rows, d.nt, d.waves, d.depth));
     return true;
   }
-  *why = "a plan is \"auto\", \"tile RT NT WM WN PW KW PARTS\", \"streaming DEPTH NT MT WAVES ROWS SPLIT\" or \"decode ROWS NT WAVES DEPTH\"";
+  *why = "a plan is \"auto\", \"tile RT NT WM WN PW KW PARTS [BANDS]\", \"streaming DEPTH NT MT WAVES ROWS SPLIT\" or \"decode ROWS NT WAVES DEPTH\"";
   return false;
 }
 
@@ -568,6 +570,10 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
       text = "tile: " + std::to_string(32 * t.rt * t.wm) + " x " + std::to_string(32 * t.nt * t.wn) + ", " +
              std::to_string(t.wm * t.wn * t.kw) + " + " + std::to_string(t.pw) + " waves" +
              (t.kw > 1 ? " (the computing waves split the k tile)" : "") + ", " + std::to_string(t.tiles) + " tiles";
+      if (t.xcd_rows != 0) {
+        const int rows = static_cast<int>(blkq4::ceil_div(m, 32 * t.rt * t.wm)) / t.xcd_rows;
+        text += ", blocks of " + std::to_string(rows) + " x " + std::to_string(32 / rows) + " tiles per XCD";
+      }
       if (t.split_k > 1) {
         text += ", the last " + std::to_string(t.split_tiles) + " in " + std::to_string(t.split_k) + " parts (workspace " +
                 std::to_string(t.workspace_bytes) + " bytes)";

@@ -457,6 +457,52 @@ inline size_t tile_workspace_bytes(const TileShape& t) {
   return kCounterBytes + static_cast<size_t>(t.split_tiles) * t.split_k * tile_elems * 4;
 }
 
+// Tile order inside a whole round of 256 unsplit tiles.  Workgroup w of a round runs on XCD w % 8 (round-robin
+// dispatch), each XCD with an L2 of its own.  In the column-major tile order an XCD gets every eighth tile: with 8 or
+// more tile rows that is m_tiles / 8 rows x ALL the round's columns.  xcd_rows = 1, 2, 4 or 8 cuts the round's
+// m_tiles x (256 / m_tiles) rectangle into xcd_rows row bands x (8 / xcd_rows) column bands instead, one block per
+// XCD.  Needs m_tiles to be a power of two between xcd_rows and 32 * xcd_rows.  The kernel's argument: log2 of
+// xcd_rows, of the block's rows and of the round's columns, 4 bits each.
+inline int log2_exact(int v) {
+  int l = 0;
+  while ((1 << l) < v) ++l;
+  return (1 << l) == v ? l : -1;
+}
+inline bool xcd_tile_map(int m_tiles, int xcd_rows, int* map) {
+  const int ml = log2_exact(m_tiles), xl = log2_exact(xcd_rows);
+  if (ml < 0 || xl < 0 || ml > 8 || xl > 3 || xl > ml || ml - xl > 5) return false;
+  *map = xl | (ml - xl) << 4 | (8 - ml) << 8 | 1 << 12;
+  return true;
+}
+
+// Which cut to use: per k, the 32 tiles of an XCD make its L2 fetch (block rows) x 2 BM + (block columns) x BN / 2
+// bytes.  Blocks are used when they fetch at most 0.6 of what every-eighth-tile fetches.  Measured with forced plans
+// (same process, us; 0 = every eighth tile, else xcd_rows): M = 512, K = N = 4096 in 64 x 128 tiles (8 tile rows: a whole
+// row of 32 tiles per XCD, 71 MB through the fabric; 2 row bands make it 33 MB) 23.4 | 1: 22.6, 2: 21.6, 4: 22.3, 8: 23.0;
+// nothing else moves by more than 1 %: M = 1024 in 128 x 128 tiles 33.6 | 33.5 - 33.9, C4 58.0 | 58.2 - 59.0,
+// M = 512, N = 11008 in 128 x 128 tiles 53.9 | 53.1 - 54.2, M = 1024, K = N = 8192 114.0 | 112.6 - 114.0, C5 1500 - 1527 |
+// 1500 - 1516.
+inline int xcd_rows_for(const TileShape& t, int m) {
+  const int bm = 32 * t.rt * t.wm, bn = 32 * t.nt * t.wn;
+  const int m_tiles = static_cast<int>(ceil_div(m, bm));
+  const int ml = log2_exact(m_tiles);
+  if (ml < 0 || ml > 8 || t.tiles - t.split_tiles < kComputeUnits) return 0;
+  auto fetched = [&](int xcd_rows) {
+    const int rows = m_tiles / xcd_rows;
+    return rows * bm * 4 + (32 / rows) * bn;
+  };
+  const int as_is = fetched(m_tiles < 8 ? m_tiles : 8);
+  int best = 0, best_bytes = as_is;
+  for (int xr = 1; xr <= 8 && xr <= m_tiles; xr *= 2) {
+    if (m_tiles / xr > 32) continue;
+    if (fetched(xr) < best_bytes) {
+      best = xr;
+      best_bytes = fetched(xr);
+    }
+  }
+  return best_bytes * 10 <= as_is * 6 ? best : 0;
+}
+
 // Measured microseconds per 64-deep k tile of one workgroup when `busy` workgroups share the chip (fp16, blocks
 // of 64 along K, K = N = 4096 ... 11008): flat while half the compute units idle, then rising with the load
 // on the memory system and the clock the chip holds -- 64 x 128: 0.29 (<= 192 workgroups) to 0.36 (256),
@@ -592,6 +638,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
       }
     }
   }
+  best.xcd_rows = xcd_rows_for(best, m);
   return best;
 }
 

@@ -63,10 +63,13 @@ typedef struct {
  * kw = 4 (with wm = wn = 1): four computing waves share the one (32 rt) x (32 nt) tile and split every 64-deep k tile
  * between them; kw = 1 otherwise.
  * split_k > 1: the last split_tiles tiles of the tile order are computed by split_k workgroups each, which
- * leave fp32 partial tiles in the workspace; the last of them to finish sums them in a fixed order. */
+ * leave fp32 partial tiles in the workspace; the last of them to finish sums them in a fixed order.
+ * xcd_rows: 0, or into how many row bands (1, 2, 4 or 8) a round of 256 tiles is cut for the 8 XCDs, each of which then
+ * owns one band x (xcd_rows / 8 of the round's columns) -- see xcd_tile_map() in blkq4_choose.h. */
 typedef struct {
   int rt, nt, wm, wn, pw;
   int kw;
+  int xcd_rows;
   int split_k;            /* 1: no workspace needed */
   int split_tiles;        /* 0 without a split */
   int tiles;              /* all tiles of the problem */

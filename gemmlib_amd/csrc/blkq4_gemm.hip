@@ -145,7 +145,7 @@ __global__ __launch_bounds__(64 * (WM * WN * KW + PW))
         const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ S,
         const uint8_t* __restrict__ Z, uint16_t* __restrict__ C, const uint16_t* __restrict__ bias, int M, int N,
         int K, int m_tiles, int whole_tiles, int split_tiles, int split_k, float* __restrict__ partials,
-        int* __restrict__ counters) {
+        int* __restrict__ counters, int xcd_map) {
   using St = Stage<BS, RT, NT, WM, WN, PW, ROW, KW>;
   constexpr int kComputeWaves = WM * WN * KW;
   constexpr bool KS = KW > 1;
@@ -188,8 +188,17 @@ __global__ __launch_bounds__(64 * (WM * WN * KW + PW))
     part = u / split_tiles;
     parts = split_k;
   }
-  const int bm = tile % m_tiles;
-  const int bn = tile / m_tiles;
+  int bm = tile % m_tiles;
+  int bn = tile / m_tiles;
+  if (xcd_map != 0 && tile < (whole_tiles & ~255)) {
+    // A whole round of 256 unsplit tiles (256 / m_tiles tile columns): workgroup w of the round runs on XCD w % 8, and
+    // the 32 tiles of an XCD are made a block of (1 << rp) tile rows x (32 >> rp) tile columns, so that its L2 fetches
+    // fewer rows and weights than with every eighth tile of the column-major order (encoding: xcd_tile_map()).
+    const int xm = xcd_map & 15, rp = (xcd_map >> 4) & 15, cl = (xcd_map >> 8) & 15;
+    const int wl = tile & 255, x = wl & 7, j = wl >> 3;
+    bm = ((x & ((1 << xm) - 1)) << rp) + (j & ((1 << rp) - 1));
+    bn = ((tile >> 8) << cl) + ((x >> xm) << (5 - rp)) + (j >> rp);
+  }
   const int m0 = bm * kBM;
   const int nw0 = bn * kBN + wn * (32 * NT);
   // N is a multiple of 32, so 32-column fragments are whole; a fragment past the end re-reads the last one
@@ -908,6 +917,9 @@ int launch_one(const blkq4_gemm_args* a) {
     partials = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + kCounterBytes);
   }
   if (t.tiles != tiles) return static_cast<int>(hipErrorInvalidValue);
+  // the tile order inside whole rounds: 0 (every eighth tile of the column-major order per XCD) or blocks
+  int xcd_map = 0;
+  if (t.xcd_rows != 0 && !xcd_tile_map(m_tiles, t.xcd_rows, &xcd_map)) return static_cast<int>(hipErrorInvalidValue);
   if (a->dry_run) return 0;
   const dim3 grid(static_cast<unsigned>(whole + split_tiles * split_k));
   // the launch's own status: a sticky error of an earlier, unrelated call stays where it is
@@ -917,7 +929,7 @@ int launch_one(const blkq4_gemm_args* a) {
                                         static_cast<const uint8_t*>(a->scales),
                                         static_cast<const uint8_t*>(a->zero_points), static_cast<uint16_t*>(a->c),
                                         static_cast<const uint16_t*>(a->bias), a->m, a->n, a->k, m_tiles, whole,
-                                        split_tiles, split_k, partials, counters));
+                                        split_tiles, split_k, partials, counters, xcd_map));
 }
 
 // The tile shapes that exist, (RT, NT, WM, WN, PW): what blkq4::choose() may ask for.  Those with whole rows

@@ -272,9 +272,12 @@ int blkq4_gemm_plan_sm80(
  * blkq4_fp16_gemm_sm80 / blkq4_bf16_gemm_sm80 (bf16 != 0) with the kernel given by the caller instead of the library's
  * cost model.  `plan` is text:
  *   "auto"                                     what the cost model picks (then identical to the entry points above);
- *   "tile RT NT WM WN PW KW PARTS"             the tile kernel: WM x WN computing waves of (32 RT) x (32 NT) outputs, PW
+ *   "tile RT NT WM WN PW KW PARTS [BANDS]"     the tile kernel: WM x WN computing waves of (32 RT) x (32 NT) outputs, PW
  *                                              producer waves, KW = 4 for the tiles whose waves split the k tile (else
  *                                              1), the tiles of the last round shared out over PARTS workgroups along K;
+ *                                              BANDS (optional; 1, 2, 4 or 8): every whole round of 256 tiles is dealt to
+ *                                              the 8 XCDs in blocks, BANDS row bands x 8 / BANDS column bands; 0 or
+ *                                              absent: every eighth tile of the column-major order per XCD;
  *   "streaming DEPTH NT MT WAVES ROWS SPLIT"   the weight-streaming kernel: slices in flight, column tiles and row tiles
  *                                              (1: up to 16 rows, 2: row groups of 32) per workgroup, waves, rows whole
  *                                              in LDS (1) or staged per slice (2), SPLIT = WAVES or 1;

@@ -297,6 +297,11 @@ def test_non_default_stream(oracle, capi, device):
     (200, 2048, 2048, ["auto", "tile 2 1 1 4 4 1 1", "tile 4 1 1 4 4 1 1", "tile 4 1 1 4 4 1 2", "tile 4 2 1 4 4 1 1",
                        "tile 8 2 1 4 0 1 1", "tile 8 1 1 4 4 1 1", "tile 4 1 1 1 4 4 1", "streaming 2 4 2 8 1 8",
                        "streaming 2 2 2 8 2 8"]),
+    # one whole round of 256 tiles plus a partly filled one (8 x 33 and 4 x 65 tiles): the tile order of the whole
+    # round in every cut per XCD, alone and with the rest split; 8 row bands do not exist for 4 tile rows
+    (512, 4224, 256, ["auto", "tile 2 1 1 4 4 1 1 0", "tile 2 1 1 4 4 1 1 1", "tile 2 1 1 4 4 1 1 2", "tile 2 1 1 4 4 1 1 4",
+                      "tile 2 1 1 4 4 1 1 8", "tile 2 1 1 4 4 1 2 2", "tile 4 1 1 4 4 1 1 1", "tile 4 1 1 4 4 1 1 2",
+                      "tile 4 1 1 4 4 1 1 4", "tile 4 1 1 4 4 1 2 4"]),
 ])
 def test_every_plan_given_as_text_is_exact_on_reference_construction(oracle, capi, device, m, n, k, plans):
     """blkq4_gemm_with_plan_sm80: whichever kernel is asked for by name, the reference's exact construction
@@ -315,3 +320,5 @@ def test_every_plan_given_as_text_is_exact_on_reference_construction(oracle, cap
         assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16)), plan
     with pytest.raises(capi.Blkq4Error, match="Kernel execution failed: invalid argument"):
         capi.gemm_with_plan("decode 16 1 8 2", bs, True, m, n, k, a_dev, q_w, q_s, q_zp, out)   # K is not 16 slices
+    with pytest.raises(capi.Blkq4Error, match="Kernel execution failed: invalid argument"):
+        capi.gemm_with_plan("tile 4 1 1 4 4 1 1 3", bs, True, m, n, k, a_dev, q_w, q_s, q_zp, out)  # no such cut

@@ -59,7 +59,7 @@ def test_split_plans_are_well_formed(capi):
     for m, n, k in itertools.product([65, 100, 128, 200, 256, 300, 512, 768, 1280], [2048, 4096, 5120, 8192, 11008, 14336, 28672],
                                      [1024, 4096, 5120, 8192, 11008, 14336, 28672]):
         text = capi.gemm_plan(64, True, m, n, k)[2]
-        got = re.match(r"tile: (\d+) x (\d+), \d \+ \d waves, (\d+) tiles, the last (\d+) in (\d+) parts \(workspace (\d+) bytes\)", text)
+        got = re.match(r"tile: (\d+) x (\d+), \d \+ \d waves, (\d+) tiles(?:, blocks of \d+ x \d+ tiles per XCD)?, the last (\d+) in (\d+) parts \(workspace (\d+) bytes\)", text)
         if not got:
             continue
         seen += 1
@@ -69,6 +69,25 @@ def test_split_plans_are_well_formed(capi):
         assert (k // 64) // parts >= 4                                     # every part has at least 4 k tiles
         assert ws == 16384 + split_tiles * parts * bm * bn * 4 <= 16384 + (32 << 20)
     assert seen > 50
+
+
+def test_tile_order_in_blocks_per_xcd_is_well_formed(capi):
+    """whole rounds of 256 tiles may be dealt to the 8 XCDs in blocks of rows x columns tiles: 32 tiles each, the rows a
+    power of two that divides the problem's tile rows (the launcher's dry run has accepted every such plan)"""
+    import re
+    assert capi.gemm_plan(64, True, 512, 4096, 4096)[2] == "tile: 64 x 128, 4 + 4 waves, 256 tiles, blocks of 4 x 8 tiles per XCD"
+    assert "XCD" not in capi.gemm_plan(64, True, 2048, 4096, 4096)[2]      # 2 x 16 as it is, 4 x 8 fetches 0.8 of that
+    seen = 0
+    for m, n, k in itertools.product([200, 256, 384, 512, 1024, 2048, 4096], [4096, 8192, 11008, 14336, 28672], [4096, 8192]):
+        text = capi.gemm_plan(64, True, m, n, k)[2]
+        got = re.match(r"tile: (\d+) x (\d+), \d \+ \d waves, (\d+) tiles, blocks of (\d+) x (\d+) tiles per XCD", text)
+        if not got:
+            continue
+        seen += 1
+        bm, bn, tiles, rows, cols = map(int, got.groups())
+        m_tiles = -(-m // bm)
+        assert rows * cols == 32 and m_tiles % rows == 0 and m_tiles & (m_tiles - 1) == 0 and tiles >= 256, text
+    assert seen >= 5
 
 
 def test_plan_rejects_what_the_gemm_rejects(capi):
