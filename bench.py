@@ -87,12 +87,12 @@ DESCRIPTION = {
 # figure of a workload is reported only while the library still picks the kernel it was taken from (TRAFFIC_KERNEL).
 COUNTER_SCALE = {"FETCH_SIZE": 131072.0 / 65552.0, "WRITE_SIZE": 1.0}
 COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
-    "C4": (44132.6, 16387.0),
+    "C4": (34411.6, 16388.8),
     "C2": (4406.1, 8.0),
     "C3": (13653.7, 344.0),
     "C5": (860380.2, 229382.3),
     "C5_prepack": (229410.8, 157706.9),
-    "C4r": (44141.1, 16385.9),
+    "C4r": (34415.1, 16386.6),
     "C2r": (4428.1, 8.0),
     "C1": (869.0, 128.0),
     "M128": (8649.1, 1024.0),
@@ -102,7 +102,7 @@ COUNTER_KIB = {  # name: (FETCH_SIZE, WRITE_SIZE)
     "M256K11K": (43374.1, 19434.3),
     "V128K": (136348.8, 250.8),
     "B16": (64097.7, 896.0),
-    "C4b": (44164.5, 16387.0),
+    "C4b": (34440.5, 16387.2),
     "C2b": (4418.6, 8.0),
 }
 
@@ -111,14 +111,14 @@ TRAFFIC_KERNEL = {  # what blkq4_gemm_plan_sm80 said the workload runs when its 
     "C1": "streaming: 8 waves splitting K, 1 column tile(s) x 32 rows, 2 slices in flight, rows whole in LDS, 2 row group(s), 128 workgroups",
     "C2": "decode: 8 waves splitting K, 4 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
     "C3": "decode: 8 waves splitting K, 4 slices requested by each, 3 column tile(s) x 16 row(s), 230 workgroups",
-    "C4": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
+    "C4": "tile: 128 x 256, 4 + 4 waves, 256 tiles, blocks of 4 x 8 tiles per XCD",
     "C5": "tile: 256 x 256, 4 + 0 waves, 1792 tiles",
-    "C4r": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
+    "C4r": "tile: 128 x 256, 4 + 4 waves, 256 tiles, blocks of 4 x 8 tiles per XCD",
     "C2r": "decode (blocks along N): 4 waves splitting K, 8 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
     "M128": "streaming: 8 waves splitting K, 4 column tile(s) x 32 rows, 2 slices in flight, rows staged per slice, 4 row group(s), 256 workgroups",
     "V128K": "decode: 8 waves splitting K, 4 slices requested by each, 2 column tile(s) x 1 row(s), 4008 workgroups",
     "B16": "streaming: 8 waves splitting K, 7 column tile(s) x 16 rows, 2 slices in flight, rows staged per slice, 1 row group(s), 256 workgroups",
-    "C4b": "tile: 128 x 256, 4 + 4 waves, 256 tiles",
+    "C4b": "tile: 128 x 256, 4 + 4 waves, 256 tiles, blocks of 4 x 8 tiles per XCD",
     "C2b": "decode: 8 waves splitting K, 4 slices requested by each, 1 column tile(s) x 1 row(s), 256 workgroups",
     "M256": "tile: 128 x 32, 4 + 4 waves (the computing waves split the k tile), 256 tiles",
     "M512": "tile: 64 x 128, 4 + 4 waves, 256 tiles, blocks of 4 x 8 tiles per XCD",

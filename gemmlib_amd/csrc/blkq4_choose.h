@@ -476,7 +476,8 @@ inline bool xcd_tile_map(int m_tiles, int xcd_rows, int* map) {
 }
 
 // Which cut to use: per k, the 32 tiles of an XCD make its L2 fetch (block rows) x 2 BM + (block columns) x BN / 2
-// bytes.  Blocks are used when they fetch at most 0.6 of what every-eighth-tile fetches.  Measured with forced plans
+// bytes.  Blocks are used when they fetch at most 0.8 of what every-eighth-tile fetches (the large tiles' time does
+// not depend on it, the traffic through the fabric does: C4 fetches 66 instead of 83 MB).  Measured with forced plans
 // (same process, us; 0 = every eighth tile, else xcd_rows): M = 512, K = N = 4096 in 64 x 128 tiles (8 tile rows: a whole
 // row of 32 tiles per XCD, 71 MB through the fabric; 2 row bands make it 33 MB) 23.4 | 1: 22.6, 2: 21.6, 4: 22.3, 8: 23.0;
 // nothing else moves by more than 1 %: M = 1024 in 128 x 128 tiles 33.6 | 33.5 - 33.9, C4 58.0 | 58.2 - 59.0,
@@ -500,7 +501,7 @@ inline int xcd_rows_for(const TileShape& t, int m) {
       best_bytes = fetched(xr);
     }
   }
-  return best_bytes * 10 <= as_is * 6 ? best : 0;
+  return best_bytes * 10 <= as_is * 8 ? best : 0;
 }
 
 // Measured microseconds per 64-deep k tile of one workgroup when `busy` workgroups share the chip (fp16, blocks

@@ -76,7 +76,8 @@ def test_tile_order_in_blocks_per_xcd_is_well_formed(capi):
     power of two that divides the problem's tile rows (the launcher's dry run has accepted every such plan)"""
     import re
     assert capi.gemm_plan(64, True, 512, 4096, 4096)[2] == "tile: 64 x 128, 4 + 4 waves, 256 tiles, blocks of 4 x 8 tiles per XCD"
-    assert "XCD" not in capi.gemm_plan(64, True, 2048, 4096, 4096)[2]      # 2 x 16 as it is, 4 x 8 fetches 0.8 of that
+    assert capi.gemm_plan(64, True, 2048, 4096, 4096)[2].endswith("blocks of 4 x 8 tiles per XCD")   # 0.8 of what 2 x 16 fetch
+    assert "XCD" not in capi.gemm_plan(16, True, 4096, 28672, 8192)[2]     # 2 x 16 and 4 x 8 of its tiles fetch the same
     seen = 0
     for m, n, k in itertools.product([200, 256, 384, 512, 1024, 2048, 4096], [4096, 8192, 11008, 14336, 28672], [4096, 8192]):
         text = capi.gemm_plan(64, True, m, n, k)[2]
