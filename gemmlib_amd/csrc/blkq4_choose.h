@@ -505,19 +505,20 @@ inline int xcd_rows_for(const TileShape& t, int m) {
 }
 
 // Measured microseconds per 64-deep k tile of one workgroup when `busy` workgroups share the chip (fp16, blocks
-// of 64 along K, K = N = 4096 ... 11008): flat while half the compute units idle, then rising with the load
-// on the memory system and the clock the chip holds -- 64 x 128: 0.29 (<= 192 workgroups) to 0.36 (256),
-// 128 x 128: 0.37 (<= 128) to 0.575, 128 x 256: 0.65 (<= 128) to 0.945, 256 x 256: 1.2 (<= 128) to 1.72 --
-// and what a workgroup spends outside its main loop.
+// of 64 along K, K = 4096 ... 14336, N = 4096 ... 28672): flat while half the compute units idle, then rising with the
+// load on the memory system and the clock the chip holds -- 64 x 128: 0.29 (<= 192 workgroups) to 0.33 (256),
+// 128 x 128: 0.32 (<= 128) to 0.51, 128 x 256: 0.65 (<= 128) to 0.89, 256 x 256: 1.07 (<= 128) to 1.63 --
+// and what a workgroup spends outside its main loop.  (Refitted after the loops were unrolled and the tiles dealt to
+// the XCDs in blocks: 128 x 128 had been 0.37 to 0.575 and lost M = 384 ... 512 at K = 11008 to slower plans by 10 %.)
 struct TileCost {
   double step_idle, step_slope, fixed;
   int flat_until;
 };
 inline TileCost tile_cost(const TileShape& t) {
-  if (t.rt == 8) return {1.20, 0.0041, 3.0, 128};
-  if (t.rt == 4 && t.nt == 2) return {0.65, 0.0023, 2.0, 128};
-  if (t.rt == 4) return {0.37, 0.0016, 1.5, 128};
-  if (t.rt == 2 && t.wn == 4) return {0.29, 0.0011, 1.0, 192};
+  if (t.rt == 8) return {1.07, 0.0044, 3.0, 128};
+  if (t.rt == 4 && t.nt == 2) return {0.65, 0.0019, 2.0, 128};
+  if (t.rt == 4) return {0.32, 0.0015, 2.0, 128};
+  if (t.rt == 2 && t.wn == 4) return {0.29, 0.00065, 1.0, 192};
   return {0.55, 0.0, 0.0, 256};  // tiles of one row tile (up to 64 rows)
 }
 inline double tile_round_us(const TileShape& t, int k_tiles, long busy) {
@@ -539,9 +540,12 @@ inline double k_split_waves_estimate_us(const TileShape& t, int k) {
 
 // Estimated time of the tile kernel with shape t (split or not) on k: whole rounds of unsplit tiles, a last
 // round of what is left of them, then one round of parts: their share of the k tiles, the partial tile
-// written once and all parts read by the workgroup that arrives last (about 100 GB/s) plus 4 us for the cache
+// written once and all parts read by the workgroup that arrives last (about 100 GB/s) plus 5 us for the cache
 // write-back and invalidate and the two extra barriers (measured: 64 x 128 in 2 parts 17.7 - 19.1 us against
-// 18.7 unsplit at M = 256, K = N = 4096; 128 x 128 in 3 parts 32.7 against 44.6 us at K = 11008).
+// 18.7 unsplit at M = 256, K = N = 4096; 128 x 128 in 3 parts 32.7 against 44.6 us at K = 11008).  Partial tiles of more
+// than 24 MB in all no longer stay in the eight L2s (32 MB) until they are summed: 128 x 256 tiles in 4 parts on every
+// compute unit (33.5 MB) take 7 us longer than the rest of the formula says (M = 512, N = 4096, K = 11008: 57.7 us, in
+// 3 parts 56.2, 128 x 128 tiles in 2 parts 52.5).
 inline double tile_estimate_us(const TileShape& t, int k) {
   if (t.kw > 1) return k_split_waves_estimate_us(t, k);
   const int kt = k / 64;
@@ -552,7 +556,9 @@ inline double tile_estimate_us(const TileShape& t, int k) {
     const long units = static_cast<long>(t.split_tiles) * t.split_k;
     const double tile_bytes = 4.0 * (32 * t.rt * t.wm) * (32 * t.nt * t.wn);
     us += static_cast<double>(ceil_div(units, kComputeUnits)) *
-          (tile_round_us(t, static_cast<int>(ceil_div(kt, t.split_k)), units) + 4.0 + (1 + t.split_k) * tile_bytes / 100e3);
+          (tile_round_us(t, static_cast<int>(ceil_div(kt, t.split_k)), units) + 5.0 + (1 + t.split_k) * tile_bytes / 100e3);
+    const double partial_bytes = static_cast<double>(units) * tile_bytes;
+    if (partial_bytes > 24e6) us += (partial_bytes - 24e6) / 1.36e6;
   }
   return us;
 }
@@ -632,8 +638,8 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
       t.workspace_bytes = tile_workspace_bytes(t);
       if (t.workspace_bytes > workspace_capacity || static_cast<size_t>(rem) * sizeof(int) > kCounterBytes) continue;
       const double us = tile_estimate_us(t, k);
-      // a split has to promise a tenth less than the best unsplit shape: its estimate is the less certain one
-      if (us < 0.9 * best_unsplit_us && us < best_us) {
+      // a split has to promise a twentieth less than the best unsplit shape: its estimate is the less certain one
+      if (us < 0.95 * best_unsplit_us && us < best_us) {
         best = t;
         best_us = us;
       }
