@@ -224,6 +224,19 @@ def test_every_m_band(oracle, capi, device, m, bs, has_offsets):
     run_gaussian(oracle, capi, device, bs, has_offsets, m, 352, 512, seed=m * 10 + bs)
 
 
+# whole rounds of tiles dealt to the XCDs in blocks (the plan says so): one round, several rounds with a partly filled
+# last one, rows that end inside the last tile row, every tile shape that takes blocks
+XCD_BLOCK_CASES = [(64, True, 2048, 11008, 512), (32, True, 512, 4096, 512), (16, True, 1024, 4096, 256),
+                   (64, True, 1000, 8192, 512), (64, False, 2048, 4096, 256)]
+
+
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", XCD_BLOCK_CASES)
+def test_tiles_in_blocks_per_xcd_on_gaussian_data(oracle, capi, device, bs, has_offsets, m, n, k):
+    assert "tiles per XCD" in capi.gemm_plan(bs, True, m, n, k, has_offsets)[2]
+    # every row and column is checked where the oracle takes a second or two, else 40 rows spread over all tile rows
+    run_gaussian(oracle, capi, device, bs, has_offsets, m, n, k, seed=m + n + k, sample_rows=None if m * n <= 2 ** 22 else 40)
+
+
 def test_rows_are_independent(oracle, capi, device):
     """row r of C depends only on row r of A: the M=1 result equals row 0 of the M=16 and M=64 results."""
     a, w = gaussian_problem(77, 64, 512, 1024)

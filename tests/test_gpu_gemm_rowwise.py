@@ -43,6 +43,8 @@ TILE_CASES = [
     (16, True, 400, 672, 576), (32, True, 1000, 4128, 128), (64, False, 1100, 4160, 192), (64, True, 640, 4160, 192),
     (16, True, 4096, 4096, 128), (32, False, 4000, 4128, 64), (64, True, 4096, 4096, 192), (16, False, 4090, 4128, 64),
     (32, True, 160, 96, 8256), (16, False, 130, 2080, 128), (32, True, 400, 2112, 128), (64, False, 300, 4160, 192),
+    # one whole round of tiles, dealt to the XCDs in blocks
+    (64, True, 2048, 4096, 192), (32, False, 1024, 4096, 128), (16, True, 512, 4096, 128),
 ]
 
 
