@@ -80,7 +80,7 @@ def candidate_plans(column_wise, m, n, k):
         slices = k // 128
         for waves in (4, 8, 16):
             depth = -(-slices // waves)
-            for nt in (1, 2, 3):
+            for nt in (1, 2, 3, 4):
                 plans.append(f"decode {rows} {nt} {waves} {depth}")
     elif m <= 1024:
         for nt in (1, 2, 4, 6, 8):

@@ -133,7 +133,11 @@ inline bool streaming_takes_few_rows(int m, int n, int k) {
 // Eight and sixteen rows keep 64 to 128 KiB of rows per workgroup, so one or two workgroups fit a compute unit and a
 // second round of them starts from nothing; once there are more rounds than that the streaming kernel, whose
 // workgroups keep their rows and walk over the column tiles, is faster (M = 16, K = 4096, N = 28672: 17.2 against
-// 20.9 us; M = 8, K = 8192, N = 14336: 15.5 against 18.4; but M = 16, K = 4096, N = 11008: 9.2 against 7.9).
+// 20.9 us; M = 8, K = 8192, N = 14336: 15.5 against 18.4; but M = 16, K = 4096, N = 11008: 9.2 against 7.9).  Sixteen rows
+// take up to four tiles per workgroup (all of LDS at K = 4096), which keeps layers of 12304 ... 16384 columns in one round:
+// M = 9 ... 16, K = 4096, N = 14336 9.1 - 9.9 us against the streaming kernel's 10.4 - 10.9, N = 16384 10.1 against 11.1 (at
+// N = 11008 three tiles stay ahead, 8.7 against 9.4); with eight rows a fourth tile gains nothing (N = 14336 8.6 against
+// 8.7 with two, N = 16384 9.6 against 9.0).
 inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) {
   if (m < 1 || m > kDecodeMaxRows || (k % 128) != 0 || (n % 16) != 0 ||
       static_cast<uint64_t>(k) * static_cast<uint64_t>(n) > (uint64_t{1} << 32)) {
@@ -169,7 +173,7 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
   }
   const int depth = (slices + waves - 1) / waves;
   if (depth > ((rows == 16) ? 4 : (rows <= 4 && waves == 16) ? kDecodeMaxDepthSixteenWaves : kDecodeMaxDepth)) return false;
-  const int max_nt = rows >= 8 ? 3 : (waves == 8 ? 2 : 1);  // the instantiations that exist
+  const int max_nt = rows == 16 ? 4 : rows == 8 ? 3 : (waves == 8 ? 2 : 1);  // the instantiations that exist
   const float per_workgroup = rows == 1 ? 0.1f : 0.5f;
   int nt = 1;
   float best = 0.f;

@@ -409,7 +409,7 @@ int launch_kernel(const blkq4_gemm_args* a) {
   BLKQ4_DECODE_DEPTHS_9_TO_14(X, 1, 1, 16) BLKQ4_DECODE_DEPTHS_9_TO_14(X, 4, 1, 16)                \
   /* eight rows fit in LDS up to K = 8192, sixteen up to K = 4096 */                               \
   BLKQ4_DECODE_DEPTHS(X, 8, 1, 8) BLKQ4_DECODE_DEPTHS(X, 8, 2, 8) BLKQ4_DECODE_DEPTHS(X, 8, 3, 8)  \
-  BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 1, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 2, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 3, 8)
+  BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 1, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 2, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 3, 8) BLKQ4_DECODE_DEPTHS_TO_4(X, 16, 4, 8)
 // blocks along N: up to four rows, one tile, K up to 8192
 #define BLKQ4_DECODE_ROW_SHAPES(X)                                                    \
   BLKQ4_DECODE_DEPTHS(X, 1, 1, 8) BLKQ4_DECODE_DEPTHS(X, 4, 1, 8)                     \

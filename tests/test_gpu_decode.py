@@ -29,11 +29,13 @@ EXACT_CASES = [
     (32, True, 3, 704, 11008), (16, True, 1, 256, 12288), (64, False, 2, 128, 14336), (64, True, 4, 32, 16384),
     (32, False, 1, 128256, 512),   # many workgroups
     (64, False, 1, 256, 28672), (32, True, 4, 128, 18432), (16, True, 2, 64, 17408),   # sixteen waves x 14, 9, 9 (uneven)
-    # five to sixteen rows: rows staged slot by slot, 1 to 3 column tiles per workgroup
+    # five to sixteen rows: rows staged slot by slot, 1 to 3 (sixteen rows: 4) column tiles per workgroup
     (32, True, 16, 11008, 4096),   # 3 tiles per workgroup, 230 workgroups, the last one with a tile missing
     (64, False, 8, 4096, 8192), (16, True, 5, 1056, 1152), (32, False, 9, 704, 512), (64, True, 16, 4128, 4096),
     (16, True, 12, 2080, 2048), (64, True, 7, 32, 1024), (32, True, 16, 128, 128), (16, False, 6, 8192, 6144),
     (64, False, 13, 8192, 3200), (32, True, 8, 28672, 1024),
+    # sixteen rows, 4 tiles per workgroup: 224 workgroups; 193 with a tile missing in the last; one and two slices per wave
+    (64, True, 16, 14336, 4096), (32, False, 9, 12320, 4096), (16, True, 12, 13312, 1024), (64, True, 10, 16384, 2176),
 ]
 
 
@@ -120,7 +122,7 @@ def test_exact_on_known_answer_construction_in_bf16(oracle, capi, device, bs, ha
 @pytest.mark.parametrize("bs,has_offsets,m,n,k", [
     (64, False, 1, 4096, 4096), (32, True, 4, 11008, 4096), (16, True, 2, 2048, 8192), (64, True, 1, 4096, 11008),
     (32, False, 3, 14336, 1152), (64, False, 1, 128256, 4096), (32, True, 16, 11008, 4096), (16, True, 8, 4096, 8192),
-    (64, True, 11, 5120, 2176),
+    (64, True, 11, 5120, 2176), (32, True, 16, 14336, 4096), (16, False, 9, 12320, 3072),
 ])
 def test_gaussian_within_tolerance_same_bits_every_call(oracle, capi, device, bs, has_offsets, m, n, k):
     a, w = gaussian_problem(5 + m + n + k, m, n, k)
@@ -137,7 +139,8 @@ def test_gaussian_within_tolerance_same_bits_every_call(oracle, capi, device, bs
         assert max_rel_err(got, other) <= 2e-3                           # fp32 sums in another order
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, True, 1, 4096, 4096), (16, True, 4, 2080, 1152), (32, True, 16, 11008, 4096)])
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, True, 1, 4096, 4096), (16, True, 4, 2080, 1152), (32, True, 16, 11008, 4096),
+                                                  (64, True, 16, 14336, 4096)])
 def test_gaussian_in_bf16(oracle, capi, device, bs, has_offsets, m, n, k):
     a, w = gaussian_bits(oracle, 77 + m + n + k, m, n, k)
     q_w, q_s, q_zp = quantize_bf16(capi, device, bs, w, has_offsets)
@@ -147,7 +150,8 @@ def test_gaussian_in_bf16(oracle, capi, device, bs, has_offsets, m, n, k):
     assert max_rel_err(oracle.bf16_to_f32(got), oracle.bf16_to_f32(ref)) <= 1e-2
 
 
-@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, False, 1, 4096, 4096), (32, True, 3, 1056, 1152), (16, True, 4, 2048, 8192), (32, True, 16, 11008, 4096)])
+@pytest.mark.parametrize("bs,has_offsets,m,n,k", [(64, False, 1, 4096, 4096), (32, True, 3, 1056, 1152), (16, True, 4, 2048, 8192), (32, True, 16, 11008, 4096),
+                                                  (64, False, 13, 14336, 4096)])
 def test_bias_in_the_epilogue_equals_a_separate_add(oracle, capi, device, bs, has_offsets, m, n, k):
     """as the reference module adds it (python/ms_blkq4linear.py:26-27): to the rounded output, in the tensor
     library's way of adding two 16-bit tensors"""
