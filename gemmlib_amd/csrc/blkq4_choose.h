@@ -198,7 +198,10 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
   if (rows >= 8) {
     const int per_unit = static_cast<size_t>(d->lds_bytes) * 2 <= kMaxLdsBytes ? 2 : 1;  // workgroups a compute unit holds
     const int rounds = ((tiles + nt - 1) / nt + kComputeUnits * per_unit - 1) / (kComputeUnits * per_unit);
-    if (rounds > per_unit) return false;
+    // (two rounds of one workgroup per unit still win while a wave requests five slices: M = 6 ... 8, K = 5120,
+    // N = 13824 and 15360 11.4 - 12.1 us against 12.7 - 13.5, the streaming kernel's rings asking for a fifth more
+    // slices than K = 5120 has; with six, K = 6144, N = 14336 and 16384, 13.8 - 14.7 against 13.0 - 14.1)
+    if (rounds > per_unit && !(rounds == 2 && depth <= 5)) return false;
   }
   return true;
 }
@@ -588,6 +591,19 @@ inline double one_row_tile_estimate_us(const TileShape& t, int k) {
   return static_cast<double>(ceil_div(t.tiles, kComputeUnits)) * (fixed + (k / 64) * step);
 }
 
+// The 64 x 128 tile on 33 to 64 rows, unsplit or every tile in parts.  Split, no two workgroups share a weight and
+// the chip's load counts for more than the general estimate says once more than 160 workgroups run: measured minus
+// estimated (fp16, blocks of 64) 0 ... -1.3 us at 128 workgroups (N = 4096, K = 4096 ... 14336 in 4 parts), 0.7 at 160,
+// 1.0 ... 1.5 at 172 ... 192 (16 ... 32 k tiles a part), 2.2 ... 2.9 at 216 ... 240, 3.0 and 4.5 at 256 (64 and 112 k
+// tiles a part).
+inline double few_rows_tile_estimate_us(const TileShape& t, int k) {
+  if (t.split_k == 1) return one_row_tile_estimate_us(t, k);
+  const long units = static_cast<long>(t.split_tiles) * t.split_k;
+  double us = tile_estimate_us(t, k);
+  if (units > 160) us += 1.5 + 0.023 * static_cast<double>(ceil_div(k / 64, t.split_k)) * static_cast<double>(units - 160) / 96.0;
+  return us;
+}
+
 // The tile kernel's plan: the shape with the smallest estimate; when its last round of tiles would leave most
 // of the chip idle and the estimate says it pays, those last `split_tiles` tiles are each shared out over
 // split_k workgroups.  Up to 64 rows with blocks along K: tiles of one row tile, which fetch every packed
@@ -603,12 +619,33 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
     t.tiles = static_cast<int>(ceil_div(m, 32 * rt * wm) * ceil_div(n, 32 * nt * wn));
     return t;
   };
+  const int kt = k / 64;
   if (column_wise && m <= 64) {
     const int rt = m <= 32 ? 1 : 2;
     const TileShape narrow = shape(rt, 1, 1, 4, 4), wide = shape(rt, 1, 1, 8, 0);
-    return one_row_tile_estimate_us(narrow, k) <= one_row_tile_estimate_us(wide, k) ? narrow : wide;
+    TileShape one = one_row_tile_estimate_us(narrow, k) <= one_row_tile_estimate_us(wide, k) ? narrow : wide;
+    if (rt == 2) {
+      // 33 to 64 rows on a layer that does not fill the chip: the 64 x 128 tile, which is the narrow shape here, has
+      // a split form (M = 64, N = 5120, K = 13824: 23.0 us in 4 parts, 30.3 streaming, 55 unsplit; N = 8192, K = 28672:
+      // 48.8, 62.9 and 110; N = 16384, K = 8192: 31.8 in 2 parts, 36.0 and 35.2)
+      const double unsplit_us = one_row_tile_estimate_us(one, k);
+      double best_us = unsplit_us;
+      TileShape t = narrow;
+      for (int split = 2; split <= kMaxSplit; ++split) {
+        if (t.tiles * split > kComputeUnits || kt / split < kMinKTilesPerPart) break;
+        t.split_k = split;
+        t.split_tiles = t.tiles;
+        t.workspace_bytes = tile_workspace_bytes(t);
+        if (t.workspace_bytes > workspace_capacity || static_cast<size_t>(t.tiles) * sizeof(int) > kCounterBytes) continue;
+        const double us = few_rows_tile_estimate_us(t, k);
+        if (us < 0.95 * unsplit_us && us < best_us) {
+          one = t;
+          best_us = us;
+        }
+      }
+    }
+    return one;
   }
-  const int kt = k / 64;
   double best_us = 0.0, best_unsplit_us = 0.0;
   for (const auto& sh : kTileShapes) {
     const TileShape t = shape(sh[0], sh[1], sh[2], sh[3], sh[4]);
@@ -676,7 +713,11 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
     // were not among them); against the tile kernel's estimate it picks the slower kernel for 0.2 % of the time
     // on them.  (M = 64, N = 18432: K = 4096 29.8 us streaming, 19.6 in tiles; K = 1024 17.2 and 8.7.  With the same
     // formula for three and four row groups M = 96, N = 8192 went to the tile kernel and took 20.1 instead of 19.4 us.)
-    const double streaming_us = 3.2 + static_cast<double>(rounds) * (0.44 + s.nt * (0.69 + 0.37 * (static_cast<double>(k) / 1024.0)));
+    // Beyond K = 8192 a column tile costs more per k than that: with four of them and two row groups K = 8192 takes
+    // 20.5 us (18.2 by the line above), 13824 30.2 (26.4), 28672 61 ... 63 (47.8), hence the square.
+    const double kk = static_cast<double>(k) / 1024.0;
+    double streaming_us = 3.2 + static_cast<double>(rounds) * (0.44 + s.nt * (0.69 + 0.37 * kk));
+    if (kk > 8.0) streaming_us += static_cast<double>(rounds) * s.nt * 0.0075 * (kk - 8.0) * (kk - 8.0);
     return streaming_us < tile_us;
   }
   // more row groups, and blocks along N (from 17 rows on: M = 32, K = 8192, N = 28672 with blocks along N takes 80 us
@@ -702,7 +743,7 @@ inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t wo
   }
   if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k);
   c.t = tile_plan(column_wise, m, n, k, workspace_capacity);
-  const double tile_us = (column_wise && m <= 64) ? one_row_tile_estimate_us(c.t, k) : tile_estimate_us(c.t, k);
+  const double tile_us = (column_wise && m <= 64) ? few_rows_tile_estimate_us(c.t, k) : tile_estimate_us(c.t, k);
   c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_us) ? kFamilyStreaming : kFamilyTile;
   return c;
 }

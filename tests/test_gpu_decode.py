@@ -36,6 +36,8 @@ EXACT_CASES = [
     (64, False, 13, 8192, 3200), (32, True, 8, 28672, 1024),
     # sixteen rows, 4 tiles per workgroup: 224 workgroups; 193 with a tile missing in the last; one and two slices per wave
     (64, True, 16, 14336, 4096), (32, False, 9, 12320, 4096), (16, True, 12, 13312, 1024), (64, True, 10, 16384, 2176),
+    # eight rows, five slices per wave: one workgroup per compute unit, two rounds of them
+    (64, True, 8, 13824, 5120), (32, False, 6, 15360, 5120),
 ]
 
 

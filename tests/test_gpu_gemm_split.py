@@ -22,6 +22,9 @@ SPLIT_CASES = [
     (64, True, True, 1280, 14336, 8192, "256 x 256", 4),
     (64, False, True, 200, 5120, 8192, "128 x 128", 3),
     (32, False, False, 100, 5120, 5120, "64 x 128", 3),
+    # 33 to 64 rows: every 64 x 128 tile in parts, where the kernel would otherwise stream the weights
+    (64, True, True, 64, 5120, 5120, "64 x 128", 4),
+    (32, True, False, 40, 13824, 5120, "64 x 128", 2),
 ]
 
 
@@ -45,7 +48,7 @@ def test_split_tiles_exact_on_reference_construction(oracle, capi, device, bs, c
         assert bad.shape[0] == 0, f"call {call}: {bad.shape[0]} of {m * n} outputs differ, first {bad[:5].tolist()}"
 
 
-@pytest.mark.parametrize("bs,col,has_offsets,m,n,k,tile,parts", SPLIT_CASES[:6:2] + SPLIT_CASES[6:7])
+@pytest.mark.parametrize("bs,col,has_offsets,m,n,k,tile,parts", SPLIT_CASES[:6:2] + SPLIT_CASES[6:7] + SPLIT_CASES[8:9])
 def test_split_tiles_gaussian_deterministic_and_with_bias(oracle, capi, device, bs, col, has_offsets, m, n, k, tile, parts):
     a, w = gaussian_problem(7 * m + n + k, m, n, k)
     q_w, q_s, q_zp = quantize_on_gpu(capi, device, bs, w, has_offsets, column_wise=col)
