@@ -198,10 +198,10 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
   if (rows >= 8) {
     const int per_unit = static_cast<size_t>(d->lds_bytes) * 2 <= kMaxLdsBytes ? 2 : 1;  // workgroups a compute unit holds
     const int rounds = ((tiles + nt - 1) / nt + kComputeUnits * per_unit - 1) / (kComputeUnits * per_unit);
-    // (two rounds of one workgroup per unit still win while a wave requests five slices: M = 6 ... 8, K = 5120,
+    // (eight rows: two rounds of one workgroup per unit still win while a wave requests five slices: M = 6 ... 8, K = 5120,
     // N = 13824 and 15360 11.4 - 12.1 us against 12.7 - 13.5, the streaming kernel's rings asking for a fifth more
     // slices than K = 5120 has; with six, K = 6144, N = 14336 and 16384, 13.8 - 14.7 against 13.0 - 14.1)
-    if (rounds > per_unit && !(rounds == 2 && depth <= 5)) return false;
+    if (rounds > per_unit && !(rounds == 2 && rows == 8 && depth == 5)) return false;
   }
   return true;
 }
@@ -251,6 +251,21 @@ inline void streaming_tiles_per_workgroup(int m, int n, int k, int* nt, int* dep
   *depth = (*nt == 1 && tiles <= 2 * kComputeUnits) ? 8 : 4;
 }
 
+// Neighbouring column groups that the streaming kernel gives to one XCD one after the other: four while a column
+// group is narrower than a 128-byte line of scales (16 columns a tile), so that the line is fetched into one L2; one
+// from four tiles per group on, which deals the column groups to the eight XCDs evenly also when there are few of them
+// (80 groups of four tiles, three row groups: in fours XCDs 0 - 3 get 36 workgroups for their 32 compute units and the
+// others 24, and the launch takes two rounds, 28.9 us at M = 96, K = N = 5120; singly every XCD gets 30).
+constexpr int streaming_neighbours(int nt, int waves, int split) { return (split == waves && nt >= 4) ? 1 : 4; }
+// Workgroups of the busiest XCD (the first one) per compute unit of it, rounded up: the rounds a launch of resident
+// workgroups, one column group each, takes.
+inline long streaming_rounds(int row_groups, int col_groups, int neighbours) {
+  const int deal = 8 * neighbours;
+  const int rest = col_groups % deal;
+  const long busiest = static_cast<long>(neighbours) * (col_groups / deal) + (rest < neighbours ? rest : neighbours);
+  return (busiest * row_groups + kComputeUnits / 8 - 1) / (kComputeUnits / 8);
+}
+
 // Launch geometry of one instantiation.  Many more workgroups than the chip holds at once: a workgroup then
 // walks over several column groups (cg, cg + cg_stride, ...) and requests the first slices of the next one
 // while it finishes the current one, so only the first column group of a workgroup waits for its weights with
@@ -269,7 +284,8 @@ inline void streaming_geometry(StreamingShape* s, bool row, int n, int k) {
                              : per_slot_bytes;
   const int group_tiles = s->nt * (s->waves / s->split);
   const int col_groups = (n / 16 + group_tiles - 1) / group_tiles;
-  int cg_stride = (col_groups + 31) / 32 * 32;  // one column group per workgroup
+  const int per_xcd_round = 8 * streaming_neighbours(s->nt, s->waves, s->split);
+  int cg_stride = (col_groups + per_xcd_round - 1) / per_xcd_round * per_xcd_round;  // one column group per workgroup
   // The partial tiles lie behind the rows when both fit (one barrier less: nobody has to wait until every wave
   // is done with the rows), else they reuse the rows' space.
   const bool separate = a_bytes + red_bytes <= kMaxLdsBytes;
@@ -311,8 +327,8 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
     if (!row) {
       double best = 0.0;
       for (const int t : {1, 2, 4, 6, 8}) {
-        const long wgs = static_cast<long>(s.row_groups) * ((n / 16 + t - 1) / t);
-        const double cost = static_cast<double>((wgs + kComputeUnits - 1) / kComputeUnits) * (3.0 + 1.73 * t);
+        const long rounds = streaming_rounds(s.row_groups, (n / 16 + t - 1) / t, streaming_neighbours(t, 8, 8));
+        const double cost = static_cast<double>(rounds) * (3.0 + 1.73 * t);
         if (t == 1 || cost < best) {
           best = cost;
           nt = t;
@@ -705,7 +721,11 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
   if (m > kStreamingMaxRows) return false;
   const long row_groups = s.row_groups;
   const long streaming_groups = row_groups * ceil_div(n / 16, s.nt);
-  const long rounds = ceil_div(streaming_groups, kComputeUnits);
+  // (row groups of 32: the waves split K, a column group is s.nt tiles)
+  const long col_groups = ceil_div(n / 16, s.nt);
+  const long rounds = s.cg_stride >= col_groups
+                          ? streaming_rounds(s.row_groups, static_cast<int>(col_groups), streaming_neighbours(s.nt, s.waves, s.split))
+                          : ceil_div(streaming_groups, kComputeUnits);
   if (column_wise && m <= 64) {
     // One or two row groups of 32, blocks along K: rounds of 256 workgroups, a workgroup's time growing with its
     // column tiles and K.  Least squares over 142 measurements (M = 24 ... 64, K = 1024 ... 4096, N = 2048 ... 32768;

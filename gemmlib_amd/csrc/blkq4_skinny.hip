@@ -148,15 +148,18 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_mfma_kernel(const uint16_t
   // consecutive XCDs (8 of them).  An XCD's workgroups take, in this order: the row groups of a column
   // group (they share its weights), then the next of four neighbouring column groups (they share the 128-byte
   // lines of the scale and zero-point rows, and their weights are contiguous), so that what is shared is
-  // fetched into that XCD's L2 once.
+  // fetched into that XCD's L2 once.  Column groups of four tiles or more hold whole lines by themselves and are
+  // dealt out singly, which keeps the XCDs level when there are few of them.
   static_assert(kSplit == kWaves || kSplit == 1, "the waves split K among all of them or not at all");
   constexpr int kTileWaves = kWaves / kSplit;  // waves (or sets of waves) with column tiles of their own
   const int col_groups = ((N >> 4) + NT * kTileWaves - 1) / (NT * kTileWaves);
   const int wg = blockIdx.x;
   const int q = wg >> 3;
   const int rg = q % row_groups;
-  int cg = 4 * ((wg & 7) + 8 * ((q / row_groups) >> 2)) + ((q / row_groups) & 3);
-  if (cg >= col_groups) return;  // the grid is rounded up to whole groups of 32 column groups
+  constexpr int kNeighbours = streaming_neighbours(NT, kWaves, kSplit);
+  const int cq = q / row_groups;
+  int cg = kNeighbours * ((wg & 7) + 8 * (cq / kNeighbours)) + (cq % kNeighbours);
+  if (cg >= col_groups) return;  // the grid is rounded up to whole groups of 8 * kNeighbours column groups
   const int m0 = rg * (16 * MT);
   const int M = min(16 * MT, M_total - m0);
   A += static_cast<size_t>(m0) * K;
@@ -608,9 +611,10 @@ int launch_kernel(const blkq4_gemm_args* a) {
   const size_t a_bytes = AM == kRowsWholeInLds ? ((((static_cast<size_t>(a->k) * 2) << p.rows_log2) + 1023) & ~size_t{1023})
                                                : kPerSlotBytes;
   constexpr int kGroupTiles = NT * (kWaves / kSplit);
+  constexpr int kXcdRound = 8 * streaming_neighbours(NT, kWaves, kSplit);  // column groups dealt to the XCDs at a time
   const int col_groups = (a->n / 16 + kGroupTiles - 1) / kGroupTiles;
   if ((1 << p.rows_log2) * p.row_groups < a->m || (MT == 1 && (1 << p.rows_log2) > 16) || (MT == 2 && p.rows_log2 != 5) ||
-      p.row_groups < 1 || p.cg_stride < 32 || (p.cg_stride % 32) != 0 || p.lds_bytes > kMaxLdsBytes ||
+      p.row_groups < 1 || p.cg_stride < kXcdRound || (p.cg_stride % kXcdRound) != 0 || p.lds_bytes > kMaxLdsBytes ||
       p.red_offset + kRedBytes > p.lds_bytes || a_bytes > p.lds_bytes || (p.red_offset != 0 && p.red_offset < a_bytes) ||
       (!refill && (p.cg_stride < col_groups || kSplit == 1)) ||
       p.grid != static_cast<uint32_t>(p.cg_stride) * static_cast<uint32_t>(p.row_groups) ||
