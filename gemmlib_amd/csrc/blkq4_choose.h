@@ -259,11 +259,14 @@ inline void streaming_tiles_per_workgroup(int m, int n, int k, int* nt, int* dep
 constexpr int streaming_neighbours(int nt, int waves, int split) { return (split == waves && nt >= 4) ? 1 : 4; }
 // Workgroups of the busiest XCD (the first one) per compute unit of it, rounded up: the rounds a launch of resident
 // workgroups, one column group each, takes.
-inline long streaming_rounds(int row_groups, int col_groups, int neighbours) {
+inline long streaming_busiest_xcd(int row_groups, int col_groups, int neighbours) {
   const int deal = 8 * neighbours;
   const int rest = col_groups % deal;
   const long busiest = static_cast<long>(neighbours) * (col_groups / deal) + (rest < neighbours ? rest : neighbours);
-  return (busiest * row_groups + kComputeUnits / 8 - 1) / (kComputeUnits / 8);
+  return busiest * row_groups;
+}
+inline long streaming_rounds(int row_groups, int col_groups, int neighbours) {
+  return (streaming_busiest_xcd(row_groups, col_groups, neighbours) + kComputeUnits / 8 - 1) / (kComputeUnits / 8);
 }
 
 // Launch geometry of one instantiation.  Many more workgroups than the chip holds at once: a workgroup then
@@ -317,18 +320,23 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
   if (m > 16) {
     // Row groups of 32 rows (two row tiles share one conversion of the weights), eight waves.  A workgroup's time
     // grows with its column tiles -- measured at K = 4096: 3.0 + 1.73 us per tile (M = 128, N = 4096 with 4, 6 and 8
-    // tiles: 11.6, 15.2, 18.5 us; with 2, in two rounds: 14.9) -- and the busiest compute unit works through
-    // ceil(workgroups / 256) of them: as many tiles per workgroup (1, 2, 4, 6, 8) as make that product smallest
-    // (M = 64, N = 11008: 344 workgroups of four tiles 21.8 us, 230 of six 15.9).  Blocks along N: 28 registers of
-    // packed weights, scales and zero-points per slot and tile, so one tile.
+    // tiles: 11.6, 15.2, 18.5 us) -- and an XCD with more workgroups than compute units takes longer than their number
+    // says: 1.45 x workgroups per unit x one workgroup's time, at least the busiest unit's whole number of them
+    // (M = 96, K = N = 4096: 3 per unit of one tile, 4.7 us
+    // each by that line, take 19.9 us, 1.5 per unit of two tiles, 6.5 us each, 14.5; N = 5152: 1.97 per unit of two tiles
+    // 20.1).  As many tiles per workgroup (1, 2, 4, 6, 8) as make that smallest (M = 64, N = 11008: 344 workgroups of
+    // four tiles 21.8 us, 230 of six 15.9; M = 96, N = 5152: two tiles 20.1, six 15.5).  Blocks along N: 28 registers
+    // of packed weights, scales and zero-points per slot and tile, so one tile.
     s.row_groups = (m + 31) / 32;
     s.rows_log2 = 5;
     int nt = 1;
     if (!row) {
       double best = 0.0;
       for (const int t : {1, 2, 4, 6, 8}) {
-        const long rounds = streaming_rounds(s.row_groups, (n / 16 + t - 1) / t, streaming_neighbours(t, 8, 8));
-        const double cost = static_cast<double>(rounds) * (3.0 + 1.73 * t);
+        const double per_unit = static_cast<double>(streaming_busiest_xcd(s.row_groups, (n / 16 + t - 1) / t, streaming_neighbours(t, 8, 8))) /
+                                (kComputeUnits / 8);
+        const double whole = static_cast<double>(static_cast<long>(per_unit + 0.999));  // the busiest unit's workgroups
+        const double cost = (per_unit <= 1.0 ? 1.0 : (1.45 * per_unit > whole ? 1.45 * per_unit : whole)) * (3.0 + 1.73 * t);
         if (t == 1 || cost < best) {
           best = cost;
           nt = t;
