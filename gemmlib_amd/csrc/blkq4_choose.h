@@ -545,15 +545,19 @@ struct TileCost {
   double step_idle, step_slope, fixed;
   int flat_until;
 };
-inline TileCost tile_cost(const TileShape& t) {
-  if (t.rt == 8) return {1.07, 0.0044, 3.0, 128};
-  if (t.rt == 4 && t.nt == 2) return {0.65, 0.0019, 2.0, 128};
-  if (t.rt == 4) return {0.32, 0.0015, 2.0, 128};
-  if (t.rt == 2 && t.wn == 4) return {0.29, 0.00065, 1.0, 192};
+// bf16 converts with more instructions per weight, which counts where the conversion is what a workgroup waits for
+// (measured against fp16 on 50 shapes, M = 128 ... 1024, every plan: 64 x 128 tiles 1.30 x up to 192 workgroups and 1.14 x
+// on a full chip, 128 x 128 1.30 and 1.12, 128 x 256 1.16 and 1.04, 256 x 256 1.09 and 1.00; the 128 x 32 tiles whose waves
+// split the k tile 0.99; the streaming kernel 1.06).
+inline TileCost tile_cost(const TileShape& t, bool bf16 = false) {
+  if (t.rt == 8) return bf16 ? TileCost{1.166, 0.00365, 3.0, 128} : TileCost{1.07, 0.0044, 3.0, 128};
+  if (t.rt == 4 && t.nt == 2) return bf16 ? TileCost{0.754, 0.00137, 2.0, 128} : TileCost{0.65, 0.0019, 2.0, 128};
+  if (t.rt == 4) return bf16 ? TileCost{0.416, 0.00123, 2.0, 128} : TileCost{0.32, 0.0015, 2.0, 128};
+  if (t.rt == 2 && t.wn == 4) return bf16 ? TileCost{0.377, 0.0, 1.0, 256} : TileCost{0.29, 0.00065, 1.0, 192};
   return {0.55, 0.0, 0.0, 256};  // tiles of one row tile (up to 64 rows)
 }
-inline double tile_round_us(const TileShape& t, int k_tiles, long busy) {
-  const TileCost c = tile_cost(t);
+inline double tile_round_us(const TileShape& t, int k_tiles, long busy, bool bf16 = false) {
+  const TileCost c = tile_cost(t, bf16);
   const long b = busy < kComputeUnits ? busy : kComputeUnits;
   return c.fixed + k_tiles * (c.step_idle + (b > c.flat_until ? (b - c.flat_until) * c.step_slope : 0.0));
 }
@@ -577,17 +581,17 @@ inline double k_split_waves_estimate_us(const TileShape& t, int k) {
 // than 24 MB in all no longer stay in the eight L2s (32 MB) until they are summed: 128 x 256 tiles in 4 parts on every
 // compute unit (33.5 MB) take 7 us longer than the rest of the formula says (M = 512, N = 4096, K = 11008: 57.7 us, in
 // 3 parts 56.2, 128 x 128 tiles in 2 parts 52.5).
-inline double tile_estimate_us(const TileShape& t, int k) {
+inline double tile_estimate_us(const TileShape& t, int k, bool bf16 = false) {
   if (t.kw > 1) return k_split_waves_estimate_us(t, k);
   const int kt = k / 64;
   const long whole = t.tiles - (t.split_k > 1 ? t.split_tiles : 0);
-  double us = static_cast<double>(whole / kComputeUnits) * tile_round_us(t, kt, kComputeUnits);
-  if (whole % kComputeUnits) us += tile_round_us(t, kt, whole % kComputeUnits);
+  double us = static_cast<double>(whole / kComputeUnits) * tile_round_us(t, kt, kComputeUnits, bf16);
+  if (whole % kComputeUnits) us += tile_round_us(t, kt, whole % kComputeUnits, bf16);
   if (t.split_k > 1) {
     const long units = static_cast<long>(t.split_tiles) * t.split_k;
     const double tile_bytes = 4.0 * (32 * t.rt * t.wm) * (32 * t.nt * t.wn);
     us += static_cast<double>(ceil_div(units, kComputeUnits)) *
-          (tile_round_us(t, static_cast<int>(ceil_div(kt, t.split_k)), units) + 5.0 + (1 + t.split_k) * tile_bytes / 100e3);
+          (tile_round_us(t, static_cast<int>(ceil_div(kt, t.split_k)), units, bf16) + 5.0 + (1 + t.split_k) * tile_bytes / 100e3);
     const double partial_bytes = static_cast<double>(units) * tile_bytes;
     if (partial_bytes > 24e6) us += (partial_bytes - 24e6) / 1.36e6;
   }
@@ -633,7 +637,7 @@ inline double few_rows_tile_estimate_us(const TileShape& t, int k) {
 // split_k workgroups.  Up to 64 rows with blocks along K: tiles of one row tile, which fetch every packed
 // weight once (128 columns with four waves and four producer waves, or 256 columns with eight waves, whichever
 // one_row_tile_estimate_us() expects to be faster: the narrow ones up to one round of them, N = 32768).
-inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspace_capacity) {
+inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspace_capacity, bool bf16 = false) {
   TileShape best{};
   auto shape = [&](int rt, int nt, int wm, int wn, int pw) {
     TileShape t{};
@@ -647,6 +651,8 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
   if (column_wise && m <= 64) {
     const int rt = m <= 32 ? 1 : 2;
     const TileShape narrow = shape(rt, 1, 1, 4, 4), wide = shape(rt, 1, 1, 8, 0);
+    // (up to 64 rows the estimates of the tile and of the streaming kernel are those of fp16 for bf16 too: the choice
+    // between them was checked in bf16 on M = 40 and 64 and was within 4 % of the best plan on every shape)
     TileShape one = one_row_tile_estimate_us(narrow, k) <= one_row_tile_estimate_us(wide, k) ? narrow : wide;
     if (rt == 2) {
       // 33 to 64 rows on a layer that does not fill the chip: the 64 x 128 tile, which is the narrow shape here, has
@@ -673,7 +679,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
   double best_us = 0.0, best_unsplit_us = 0.0;
   for (const auto& sh : kTileShapes) {
     const TileShape t = shape(sh[0], sh[1], sh[2], sh[3], sh[4]);
-    const double us = tile_estimate_us(t, k);
+    const double us = tile_estimate_us(t, k, bf16);
     if (best.rt == 0 || us < best_us) {
       best = t;
       best_us = us;
@@ -702,7 +708,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
       t.split_tiles = rem;
       t.workspace_bytes = tile_workspace_bytes(t);
       if (t.workspace_bytes > workspace_capacity || static_cast<size_t>(rem) * sizeof(int) > kCounterBytes) continue;
-      const double us = tile_estimate_us(t, k);
+      const double us = tile_estimate_us(t, k, bf16);
       // a split has to promise a twentieth less than the best unsplit shape: its estimate is the less certain one
       if (us < 0.95 * best_unsplit_us && us < best_us) {
         best = t;
@@ -721,7 +727,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
 // it has more workgroups than compute units, with whole rounds of them.
 constexpr uint64_t kStreamingMaxWeights = uint64_t{1} << 33;
 
-inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const StreamingShape& s, double tile_us) {
+inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const StreamingShape& s, double tile_us, bool bf16 = false) {
   // its offsets into the packed weights (K N / 2 bytes) are 32 bits wide (so are the other kernels': the entry points
   // refuse such problems before any kernel is chosen)
   if (static_cast<uint64_t>(k) * static_cast<uint64_t>(n) >= kStreamingMaxWeights) return false;
@@ -756,13 +762,13 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
   if (streaming_groups > kComputeUnits) {
     streaming_us *= static_cast<double>(rounds) / (static_cast<double>(streaming_groups) / kComputeUnits);
   }
+  if (bf16) streaming_us *= 1.06;
   return streaming_us < tile_us;
 }
 
 // The whole decision.  workspace_capacity: bytes of workspace the caller could hand to a split tile kernel
 // (0: none, no split).
 inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity) {
-  (void)bf16;  // the same shapes for both element types
   Choice c{};
   // few rows, blocks along K, a K that a workgroup can request at once: the decode kernel
   if (decode_shape(column_wise, m, n, k, &c.d)) {
@@ -770,9 +776,9 @@ inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t wo
     return c;
   }
   if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k);
-  c.t = tile_plan(column_wise, m, n, k, workspace_capacity);
-  const double tile_us = (column_wise && m <= 64) ? few_rows_tile_estimate_us(c.t, k) : tile_estimate_us(c.t, k);
-  c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_us) ? kFamilyStreaming : kFamilyTile;
+  c.t = tile_plan(column_wise, m, n, k, workspace_capacity, bf16);
+  const double tile_us = (column_wise && m <= 64) ? few_rows_tile_estimate_us(c.t, k) : tile_estimate_us(c.t, k, bf16);
+  c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_us, bf16) ? kFamilyStreaming : kFamilyTile;
   return c;
 }
 
