@@ -590,8 +590,13 @@ inline double tile_estimate_us(const TileShape& t, int k, bool bf16 = false) {
   if (t.split_k > 1) {
     const long units = static_cast<long>(t.split_tiles) * t.split_k;
     const double tile_bytes = 4.0 * (32 * t.rt * t.wm) * (32 * t.nt * t.wn);
+    // (256 x 256: the accumulators fill the registers and the workgroup that adds the parts up has one request in
+    // flight at a time, 30 us per part -- by timestamps 118.6 us for four parts where a 128 x 256 tile's take 7.6;
+    // M = 1280, N = 14336, K = 8192 in 256 x 256 tiles with the last 24 in 4 parts 366 us, unsplit 331, in 128 x 256 tiles
+    // with the last 48 in 4 parts 260)
+    const double bytes_per_us = t.rt == 8 ? 9e3 : 100e3;
     us += static_cast<double>(ceil_div(units, kComputeUnits)) *
-          (tile_round_us(t, static_cast<int>(ceil_div(kt, t.split_k)), units, bf16) + 5.0 + (1 + t.split_k) * tile_bytes / 100e3);
+          (tile_round_us(t, static_cast<int>(ceil_div(kt, t.split_k)), units, bf16) + 5.0 + (1 + t.split_k) * tile_bytes / bytes_per_us);
     const double partial_bytes = static_cast<double>(units) * tile_bytes;
     if (partial_bytes > 24e6) us += (partial_bytes - 24e6) / 1.36e6;
   }

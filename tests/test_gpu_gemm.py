@@ -315,6 +315,9 @@ def test_non_default_stream(oracle, capi, device):
     (512, 4224, 256, ["auto", "tile 2 1 1 4 4 1 1 0", "tile 2 1 1 4 4 1 1 1", "tile 2 1 1 4 4 1 1 2", "tile 2 1 1 4 4 1 1 4",
                       "tile 2 1 1 4 4 1 1 8", "tile 2 1 1 4 4 1 2 2", "tile 4 1 1 4 4 1 1 1", "tile 4 1 1 4 4 1 1 2",
                       "tile 4 1 1 4 4 1 1 4", "tile 4 1 1 4 4 1 2 4"]),
+    # 256 x 256 tiles in parts, which no plan of the library's own asks for (the workgroup that adds the parts up is slow
+    # with 256 accumulators): 3 x 4 tiles, the last row of them 8 rows high
+    (520, 1024, 2048, ["auto", "tile 8 2 1 4 0 1 2", "tile 8 2 1 4 0 1 4", "tile 4 2 1 4 4 1 3"]),
 ])
 def test_every_plan_given_as_text_is_exact_on_reference_construction(oracle, capi, device, m, n, k, plans):
     """blkq4_gemm_with_plan_sm80: whichever kernel is asked for by name, the reference's exact construction

@@ -19,7 +19,7 @@ SPLIT_CASES = [
     (64, True, True, 200, 5120, 8192, "128 x 128", 3),
     (16, True, True, 65, 8192, 8192, "128 x 128", 4),
     (64, True, False, 300, 28672, 8192, "128 x 256", 3),
-    (64, True, True, 1280, 14336, 8192, "256 x 256", 4),
+    (64, True, True, 1280, 14336, 8192, "128 x 256", 4),
     (64, False, True, 200, 5120, 8192, "128 x 128", 3),
     (32, False, False, 100, 5120, 5120, "64 x 128", 3),
     # 33 to 64 rows: every 64 x 128 tile in parts, where the kernel would otherwise stream the weights
