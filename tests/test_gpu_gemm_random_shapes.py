@@ -3,7 +3,8 @@
 The shapes are drawn so that every way the library splits the work is hit with ragged edges: K that ends
 inside a 128-deep slice, column tile counts that the column groups do not divide, row counts around the
 row-group and kernel switches, very wide N (waves with a column tile of their own, workgroups that walk over
-several column groups), both blockings, with and without zero-points and bias.  Bar: max relative error
+several column groups, column groups dealt singly to the XCDs), 33 to 64 rows whose tiles are split along K, both
+blockings, with and without zero-points and bias.  Bar: max relative error
 <= 1e-2 on Gaussian data, where the error of an output is measured against max(|ref|, 1e-3 * max|ref|).
 """
 
@@ -45,6 +46,24 @@ def draw_cases():
             k = int(rng.integers(1, 12)) * 64
         if col and rng.integers(0, 2):
             n += 32  # blocks along K allow any multiple of 32
+        cases.append((bs, zp, col, m, n, k, bool(rng.integers(0, 2))))
+    for i in range(24):
+        bs = int(rng.choice([16, 32, 64]))
+        col = True if i % 3 else bool(rng.integers(0, 2))
+        zp = bool(rng.integers(0, 2))
+        band = i % 3
+        if band == 0:    # 33 to 64 rows, few tiles, long K: with blocks along K every 64 x 128 tile in parts
+            m = int(rng.integers(33, 65))
+            n = int(rng.integers(8, 130)) * 64
+            k = int(rng.integers(64, 300)) * 64
+        elif band == 1:  # five to eight rows, K just above 4096, wide: two rounds of decode workgroups
+            m = int(rng.integers(5, 9))
+            n = int(rng.integers(12288 // 32, 21000 // 32)) * 32
+            k = int(rng.integers(33, 41)) * 128
+        else:            # row groups with four and more tiles per workgroup, column groups that eight does not divide
+            m = int(rng.integers(17, 200))
+            n = int(rng.integers(60, 400)) * 32
+            k = int(rng.integers(8, 100)) * 64
         cases.append((bs, zp, col, m, n, k, bool(rng.integers(0, 2))))
     return cases
 
