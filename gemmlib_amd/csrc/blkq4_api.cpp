@@ -201,12 +201,12 @@ int launch_choice(const blkq4::Choice& choice, bool bf16, const blkq4_gemm_args*
 // A plan given as text (blkq4_gemm_with_plan_sm80): the kernel family and its shape parameters, everything else
 // derived the way blkq4::choose() derives it.  Whether such a kernel exists and fits the problem is the launchers'
 // check.  Returns false and says why when the text is no plan.
-bool parse_plan(const char* text, bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity,
+bool parse_plan(const char* text, int block_size, bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity,
                 blkq4::Choice* c, std::string* why) {
   *c = blkq4::Choice{};
   int v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   if (text == nullptr || std::strcmp(text, "auto") == 0) {
-    *c = blkq4::choose(column_wise, bf16, m, n, k, workspace_capacity);
+    *c = blkq4::choose(column_wise, bf16, m, n, k, workspace_capacity, block_size);
     return true;
   }
   if (std::sscanf(text, "tile %d %d %d %d %d %d %d %d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5], &v[6], &v[7]) >= 7) {
@@ -395,12 +395,12 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
   if (plan != nullptr) {
     // a plan given by the caller (blkq4_gemm_with_plan_sm80)
     std::string why;
-    if (!parse_plan(plan, column_wise_blocking, bf16, m, n, k, capacity, &choice, &why)) {
+    if (!parse_plan(plan, block_size, column_wise_blocking, bf16, m, n, k, capacity, &choice, &why)) {
       set_error(err, "Unknown plan: " + why);
       return -1;
     }
   } else {
-    choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, capacity);
+    choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, capacity, block_size);
   }
   if (choice.family == blkq4::kFamilyTile && choice.t.split_k > 1) {
     void* workspace = nullptr;
@@ -420,7 +420,7 @@ int gemm_entry(bool bf16, int block_size, bool column_wise_blocking, int m, int 
           set_error(err, "No workspace for the split the plan asks for (blkq4_gemm_workspace_info_sm80 says why)");
           return -1;
         }
-        choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, 0);
+        choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, 0, block_size);
       } else {
         args.workspace = workspace;
         args.workspace_bytes = capacity;
@@ -529,7 +529,7 @@ extern "C" BLKQ4_EXPORT int blkq4_gemm_plan_sm80(int block_size, bool column_wis
     set_error(err, kTooLarge);
     return -1;
   }
-  const blkq4::Choice choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, blkq4_dev_workspace_capacity());
+  const blkq4::Choice choice = blkq4::choose(column_wise_blocking, bf16, m, n, k, blkq4_dev_workspace_capacity(), block_size);
   blkq4_gemm_args args{};
   args.block_size = block_size;
   args.column_wise = column_wise_blocking ? 1 : 0;

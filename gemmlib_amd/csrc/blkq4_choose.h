@@ -545,19 +545,34 @@ struct TileCost {
   double step_idle, step_slope, fixed;
   int flat_until;
 };
-// bf16 converts with more instructions per weight, which counts where the conversion is what a workgroup waits for
-// (measured against fp16 on 50 shapes, M = 128 ... 1024, every plan: 64 x 128 tiles 1.30 x up to 192 workgroups and 1.14 x
-// on a full chip, 128 x 128 1.30 and 1.12, 128 x 256 1.16 and 1.04, 256 x 256 1.09 and 1.00; the 128 x 32 tiles whose waves
-// split the k tile 0.99; the streaming kernel 1.06).
-inline TileCost tile_cost(const TileShape& t, bool bf16 = false) {
-  if (t.rt == 8) return bf16 ? TileCost{1.166, 0.00365, 3.0, 128} : TileCost{1.07, 0.0044, 3.0, 128};
-  if (t.rt == 4 && t.nt == 2) return bf16 ? TileCost{0.754, 0.00137, 2.0, 128} : TileCost{0.65, 0.0019, 2.0, 128};
-  if (t.rt == 4) return bf16 ? TileCost{0.416, 0.00123, 2.0, 128} : TileCost{0.32, 0.0015, 2.0, 128};
-  if (t.rt == 2 && t.wn == 4) return bf16 ? TileCost{0.377, 0.0, 1.0, 256} : TileCost{0.29, 0.00065, 1.0, 192};
+// The constants were fitted on fp16 with blocks of 64 along K.  The other forms convert with more instructions per
+// weight, which counts where the conversion is what a workgroup waits for; measured against that form, every plan, a k
+// step takes, up to half a chip busy and on a full chip:
+//   bf16 (50 shapes, M = 128 ... 1024): 64 x 128 tiles 1.30 and 1.14 x, 128 x 128 1.30 and 1.12, 128 x 256 1.16 and 1.04,
+//     256 x 256 1.09 and 1.00; the 128 x 32 tiles whose waves split the k tile 0.99; the streaming kernel 1.06;
+//   blocks along N (36 shapes, M = 128 ... 512): 1.24 and 1.15, 1.11 and 1.085, 1.02, 1.01 and 1.00;
+//   blocks of 16 (36 shapes): 1.16 and 1.13, 1.14 and 1.09, 1.11 and 1.06, 1.075 and 1.04 (blocks of 32: as 64).
+// A row each (bf16 before blocks along N before blocks of 16 where several apply: no measurements of the combinations).
+// With fp16's row for all, 4 of the 50, 3 of the 36 and 3 of the 36 chosen plans were more than 5 % behind the best one
+// measured (up to 30 %, 128 x 128 tiles on half the chip where a split or a larger tile wins); with their own rows 0, 1
+// and 0 by the same measurements.
+enum TileCostRow { kCostPlain = 0, kCostBf16 = 1, kCostBlocksAlongN = 2, kCostBlocksOf16 = 3 };
+inline int tile_cost_row(bool column_wise, bool bf16, int block_size) {
+  return bf16 ? kCostBf16 : !column_wise ? kCostBlocksAlongN : block_size == 16 ? kCostBlocksOf16 : kCostPlain;
+}
+inline TileCost tile_cost(const TileShape& t, int row = kCostPlain) {
+  static constexpr TileCost k256x256[4] = {{1.07, 0.0044, 3.0, 128}, {1.166, 0.00365, 3.0, 128}, {1.081, 0.00432, 3.0, 128}, {1.150, 0.00428, 3.0, 128}};
+  static constexpr TileCost k128x256[4] = {{0.65, 0.0019, 2.0, 128}, {0.754, 0.00137, 2.0, 128}, {0.663, 0.00194, 2.0, 128}, {0.7215, 0.00176, 2.0, 128}};
+  static constexpr TileCost k128x128[4] = {{0.32, 0.0015, 2.0, 128}, {0.416, 0.00123, 2.0, 128}, {0.3552, 0.00156, 2.0, 128}, {0.3648, 0.00151, 2.0, 128}};
+  static constexpr TileCost k64x128[4] = {{0.29, 0.00065, 1.0, 192}, {0.377, 0.0, 1.0, 256}, {0.3596, 0.00034, 1.0, 192}, {0.3364, 0.0006, 1.0, 192}};
+  if (t.rt == 8) return k256x256[row];
+  if (t.rt == 4 && t.nt == 2) return k128x256[row];
+  if (t.rt == 4) return k128x128[row];
+  if (t.rt == 2 && t.wn == 4) return k64x128[row];
   return {0.55, 0.0, 0.0, 256};  // tiles of one row tile (up to 64 rows)
 }
-inline double tile_round_us(const TileShape& t, int k_tiles, long busy, bool bf16 = false) {
-  const TileCost c = tile_cost(t, bf16);
+inline double tile_round_us(const TileShape& t, int k_tiles, long busy, int row = kCostPlain) {
+  const TileCost c = tile_cost(t, row);
   const long b = busy < kComputeUnits ? busy : kComputeUnits;
   return c.fixed + k_tiles * (c.step_idle + (b > c.flat_until ? (b - c.flat_until) * c.step_slope : 0.0));
 }
@@ -581,12 +596,12 @@ inline double k_split_waves_estimate_us(const TileShape& t, int k) {
 // than 24 MB in all no longer stay in the eight L2s (32 MB) until they are summed: 128 x 256 tiles in 4 parts on every
 // compute unit (33.5 MB) take 7 us longer than the rest of the formula says (M = 512, N = 4096, K = 11008: 57.7 us, in
 // 3 parts 56.2, 128 x 128 tiles in 2 parts 52.5).
-inline double tile_estimate_us(const TileShape& t, int k, bool bf16 = false) {
+inline double tile_estimate_us(const TileShape& t, int k, int row = kCostPlain) {
   if (t.kw > 1) return k_split_waves_estimate_us(t, k);
   const int kt = k / 64;
   const long whole = t.tiles - (t.split_k > 1 ? t.split_tiles : 0);
-  double us = static_cast<double>(whole / kComputeUnits) * tile_round_us(t, kt, kComputeUnits, bf16);
-  if (whole % kComputeUnits) us += tile_round_us(t, kt, whole % kComputeUnits, bf16);
+  double us = static_cast<double>(whole / kComputeUnits) * tile_round_us(t, kt, kComputeUnits, row);
+  if (whole % kComputeUnits) us += tile_round_us(t, kt, whole % kComputeUnits, row);
   if (t.split_k > 1) {
     const long units = static_cast<long>(t.split_tiles) * t.split_k;
     const double tile_bytes = 4.0 * (32 * t.rt * t.wm) * (32 * t.nt * t.wn);
@@ -596,7 +611,7 @@ inline double tile_estimate_us(const TileShape& t, int k, bool bf16 = false) {
     // with the last 48 in 4 parts 260)
     const double bytes_per_us = t.rt == 8 ? 9e3 : 100e3;
     us += static_cast<double>(ceil_div(units, kComputeUnits)) *
-          (tile_round_us(t, static_cast<int>(ceil_div(kt, t.split_k)), units, bf16) + 5.0 + (1 + t.split_k) * tile_bytes / bytes_per_us);
+          (tile_round_us(t, static_cast<int>(ceil_div(kt, t.split_k)), units, row) + 5.0 + (1 + t.split_k) * tile_bytes / bytes_per_us);
     const double partial_bytes = static_cast<double>(units) * tile_bytes;
     if (partial_bytes > 24e6) us += (partial_bytes - 24e6) / 1.36e6;
   }
@@ -642,7 +657,7 @@ inline double few_rows_tile_estimate_us(const TileShape& t, int k) {
 // split_k workgroups.  Up to 64 rows with blocks along K: tiles of one row tile, which fetch every packed
 // weight once (128 columns with four waves and four producer waves, or 256 columns with eight waves, whichever
 // one_row_tile_estimate_us() expects to be faster: the narrow ones up to one round of them, N = 32768).
-inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspace_capacity, bool bf16 = false) {
+inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspace_capacity, int row = kCostPlain) {
   TileShape best{};
   auto shape = [&](int rt, int nt, int wm, int wn, int pw) {
     TileShape t{};
@@ -684,7 +699,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
   double best_us = 0.0, best_unsplit_us = 0.0;
   for (const auto& sh : kTileShapes) {
     const TileShape t = shape(sh[0], sh[1], sh[2], sh[3], sh[4]);
-    const double us = tile_estimate_us(t, k, bf16);
+    const double us = tile_estimate_us(t, k, row);
     if (best.rt == 0 || us < best_us) {
       best = t;
       best_us = us;
@@ -713,7 +728,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
       t.split_tiles = rem;
       t.workspace_bytes = tile_workspace_bytes(t);
       if (t.workspace_bytes > workspace_capacity || static_cast<size_t>(rem) * sizeof(int) > kCounterBytes) continue;
-      const double us = tile_estimate_us(t, k, bf16);
+      const double us = tile_estimate_us(t, k, row);
       // a split has to promise a twentieth less than the best unsplit shape: its estimate is the less certain one
       if (us < 0.95 * best_unsplit_us && us < best_us) {
         best = t;
@@ -732,7 +747,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
 // it has more workgroups than compute units, with whole rounds of them.
 constexpr uint64_t kStreamingMaxWeights = uint64_t{1} << 33;
 
-inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const StreamingShape& s, double tile_us, bool bf16 = false) {
+inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const StreamingShape& s, double tile_us, int row = kCostPlain) {
   // its offsets into the packed weights (K N / 2 bytes) are 32 bits wide (so are the other kernels': the entry points
   // refuse such problems before any kernel is chosen)
   if (static_cast<uint64_t>(k) * static_cast<uint64_t>(n) >= kStreamingMaxWeights) return false;
@@ -767,13 +782,13 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
   if (streaming_groups > kComputeUnits) {
     streaming_us *= static_cast<double>(rounds) / (static_cast<double>(streaming_groups) / kComputeUnits);
   }
-  if (bf16) streaming_us *= 1.06;
+  if (row == kCostBf16) streaming_us *= 1.06;
   return streaming_us < tile_us;
 }
 
 // The whole decision.  workspace_capacity: bytes of workspace the caller could hand to a split tile kernel
 // (0: none, no split).
-inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity) {
+inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity, int block_size = 64) {
   Choice c{};
   // few rows, blocks along K, a K that a workgroup can request at once: the decode kernel
   if (decode_shape(column_wise, m, n, k, &c.d)) {
@@ -781,9 +796,10 @@ inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t wo
     return c;
   }
   if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k);
-  c.t = tile_plan(column_wise, m, n, k, workspace_capacity, bf16);
-  const double tile_us = (column_wise && m <= 64) ? few_rows_tile_estimate_us(c.t, k) : tile_estimate_us(c.t, k, bf16);
-  c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_us, bf16) ? kFamilyStreaming : kFamilyTile;
+  const int row = tile_cost_row(column_wise, bf16, block_size);
+  c.t = tile_plan(column_wise, m, n, k, workspace_capacity, row);
+  const double tile_us = (column_wise && m <= 64) ? few_rows_tile_estimate_us(c.t, k) : tile_estimate_us(c.t, k, row);
+  c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_us, row) ? kFamilyStreaming : kFamilyTile;
   return c;
 }
 
