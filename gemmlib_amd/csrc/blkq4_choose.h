@@ -257,8 +257,8 @@ inline void streaming_tiles_per_workgroup(int m, int n, int k, int* nt, int* dep
 // (80 groups of four tiles, three row groups: in fours XCDs 0 - 3 get 36 workgroups for their 32 compute units and the
 // others 24, and the launch takes two rounds, 28.9 us at M = 96, K = N = 5120; singly every XCD gets 30).
 constexpr int streaming_neighbours(int nt, int waves, int split) { return (split == waves && nt >= 4) ? 1 : 4; }
-// Workgroups of the busiest XCD (the first one) per compute unit of it, rounded up: the rounds a launch of resident
-// workgroups, one column group each, takes.
+// Workgroups on the busiest XCD (the first one, which gets most of what is left over), one column group each; and
+// those per compute unit of it, rounded up: the rounds a launch of resident workgroups takes.
 inline long streaming_busiest_xcd(int row_groups, int col_groups, int neighbours) {
   const int deal = 8 * neighbours;
   const int rest = col_groups % deal;
@@ -322,11 +322,11 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
     // grows with its column tiles -- measured at K = 4096: 3.0 + 1.73 us per tile (M = 128, N = 4096 with 4, 6 and 8
     // tiles: 11.6, 15.2, 18.5 us) -- and an XCD with more workgroups than compute units takes longer than their number
     // says: 1.45 x workgroups per unit x one workgroup's time, at least the busiest unit's whole number of them
-    // (M = 96, K = N = 4096: 3 per unit of one tile, 4.7 us
-    // each by that line, take 19.9 us, 1.5 per unit of two tiles, 6.5 us each, 14.5; N = 5152: 1.97 per unit of two tiles
-    // 20.1).  As many tiles per workgroup (1, 2, 4, 6, 8) as make that smallest (M = 64, N = 11008: 344 workgroups of
-    // four tiles 21.8 us, 230 of six 15.9; M = 96, N = 5152: two tiles 20.1, six 15.5).  Blocks along N: 28 registers
-    // of packed weights, scales and zero-points per slot and tile, so one tile.
+    // (M = 96, K = N = 4096: 3 per unit of one tile, 4.7 us each by that line, take 19.9 us, 1.5 per unit of two tiles,
+    // 6.5 us each, 14.5; N = 5152: 1.97 per unit of two tiles 20.1).  As many tiles per workgroup (1, 2, 4, 6, 8) as make
+    // that smallest (M = 64, N = 11008: 344 workgroups of four tiles 21.8 us, 230 of six 15.9; M = 96, N = 5152: two tiles
+    // 20.1, six 15.5).  Blocks along N: 28 registers of packed weights, scales and zero-points per slot and tile, so one
+    // tile.
     s.row_groups = (m + 31) / 32;
     s.rows_log2 = 5;
     int nt = 1;
