@@ -31,7 +31,10 @@ VARIANTS = {
     "fp16/bs64/along-N": (False, 64, False, True),
 }
 # the variant the constants were fitted on, for --shapes
-FITTED_VARIANTS = {"fp16/bs64": (False, 64, True, True), "fp16/bs64/sym": (False, 64, True, False)}
+FITTED_VARIANTS = {"fp16/bs64": (False, 64, True, True), "fp16/bs64/sym": (False, 64, True, False),
+                   # combinations, for --shapes
+                   "bf16/bs16": (True, 16, True, True), "bf16/bs64/along-N": (True, 64, False, True),
+                   "fp16/bs16/along-N": (False, 16, False, True), "fp16/bs32": (False, 32, True, True)}
 LAYERS = [(4096, 4096), (11008, 4096), (4096, 11008), (28672, 8192), (14336, 4096)]   # (N, K)
 ROWS = [1, 4, 8, 16, 32, 64, 128, 256, 512]
 

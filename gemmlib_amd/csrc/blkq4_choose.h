@@ -552,24 +552,38 @@ struct TileCost {
 //     256 x 256 1.09 and 1.00; the 128 x 32 tiles whose waves split the k tile 0.99; the streaming kernel 1.06;
 //   blocks along N (36 shapes, M = 128 ... 512): 1.24 and 1.15, 1.11 and 1.085, 1.02, 1.01 and 1.00;
 //   blocks of 16 (36 shapes): 1.16 and 1.13, 1.14 and 1.09, 1.11 and 1.06, 1.075 and 1.04 (blocks of 32: as 64).
-// A row each (bf16 before blocks along N before blocks of 16 where several apply: no measurements of the combinations).
-// With fp16's row for all, 4 of the 50, 3 of the 36 and 3 of the 36 chosen plans were more than 5 % behind the best one
-// measured (up to 30 %, 128 x 128 tiles on half the chip where a split or a larger tile wins); with their own rows 0, 1
-// and 0 by the same measurements.
-enum TileCostRow { kCostPlain = 0, kCostBf16 = 1, kCostBlocksAlongN = 2, kCostBlocksOf16 = 3 };
+// Where several apply the factors multiply: bf16 with blocks of 16 measures 1.50 and 1.29, 1.39 and 1.20, 1.31 and 1.11,
+// 1.20 (products: 1.51 and 1.29, 1.48 and 1.22, 1.29 and 1.10, 1.17), bf16 with blocks along N 1.72 and 1.41, 1.53 and
+// 1.27, 1.31 and 1.10, 1.10 (1.61 and 1.31, 1.44 and 1.22, 1.18 and 1.06, 1.10; 24 shapes each).
+// With fp16's constants for all, a copy of tile_plan() fed with the measured times of every plan picks a plan more than
+// 5 % behind the best one for 4 of the 50, 3 of the 36 and 3 of the 36 shapes (up to 30 %: 128 x 128 tiles on half the
+// chip where a split or a larger tile wins) and, with bf16's factors alone, for 7 and 3 of the 24 + 24 shapes of the
+// combinations; with the factors as they are here for 1, 1, 0, 0 and 0.
+enum TileCostRow { kCostPlain = 0, kCostBf16 = 1, kCostBlocksAlongN = 2, kCostBlocksOf16 = 4 };  // bits
 inline int tile_cost_row(bool column_wise, bool bf16, int block_size) {
-  return bf16 ? kCostBf16 : !column_wise ? kCostBlocksAlongN : block_size == 16 ? kCostBlocksOf16 : kCostPlain;
+  return (bf16 ? kCostBf16 : 0) | (!column_wise ? kCostBlocksAlongN : 0) | (block_size == 16 ? kCostBlocksOf16 : 0);
 }
 inline TileCost tile_cost(const TileShape& t, int row = kCostPlain) {
-  static constexpr TileCost k256x256[4] = {{1.07, 0.0044, 3.0, 128}, {1.166, 0.00365, 3.0, 128}, {1.081, 0.00432, 3.0, 128}, {1.150, 0.00428, 3.0, 128}};
-  static constexpr TileCost k128x256[4] = {{0.65, 0.0019, 2.0, 128}, {0.754, 0.00137, 2.0, 128}, {0.663, 0.00194, 2.0, 128}, {0.7215, 0.00176, 2.0, 128}};
-  static constexpr TileCost k128x128[4] = {{0.32, 0.0015, 2.0, 128}, {0.416, 0.00123, 2.0, 128}, {0.3552, 0.00156, 2.0, 128}, {0.3648, 0.00151, 2.0, 128}};
-  static constexpr TileCost k64x128[4] = {{0.29, 0.00065, 1.0, 192}, {0.377, 0.0, 1.0, 256}, {0.3596, 0.00034, 1.0, 192}, {0.3364, 0.0006, 1.0, 192}};
-  if (t.rt == 8) return k256x256[row];
-  if (t.rt == 4 && t.nt == 2) return k128x256[row];
-  if (t.rt == 4) return k128x128[row];
-  if (t.rt == 2 && t.wn == 4) return k64x128[row];
-  return {0.55, 0.0, 0.0, 256};  // tiles of one row tile (up to 64 rows)
+  // 64 x 128, 128 x 128, 128 x 256, 256 x 256
+  static constexpr TileCost kPlain[4] = {{0.29, 0.00065, 1.0, 192}, {0.32, 0.0015, 2.0, 128}, {0.65, 0.0019, 2.0, 128}, {1.07, 0.0044, 3.0, 128}};
+  // factors on the k step of (up to flat_until workgroups, 256 workgroups) for bf16, blocks along N, blocks of 16
+  static constexpr double kFactor[3][4][2] = {{{1.30, 1.14}, {1.30, 1.12}, {1.16, 1.04}, {1.09, 1.00}},
+                                              {{1.24, 1.15}, {1.11, 1.085}, {1.02, 1.02}, {1.01, 1.00}},
+                                              {{1.16, 1.13}, {1.14, 1.09}, {1.11, 1.06}, {1.075, 1.04}}};
+  const int shape = t.rt == 8 ? 3 : (t.rt == 4 && t.nt == 2) ? 2 : t.rt == 4 ? 1 : (t.rt == 2 && t.wn == 4) ? 0 : -1;
+  if (shape < 0) return {0.55, 0.0, 0.0, 256};  // tiles of one row tile (up to 64 rows)
+  TileCost c = kPlain[shape];
+  if (row == kCostPlain) return c;
+  double idle = c.step_idle, full = c.step_idle + (kComputeUnits - c.flat_until) * c.step_slope;
+  for (int bit = 0; bit < 3; ++bit) {
+    if (row & (1 << bit)) {
+      idle *= kFactor[bit][shape][0];
+      full *= kFactor[bit][shape][1];
+    }
+  }
+  c.step_idle = idle;
+  c.step_slope = full > idle ? (full - idle) / (kComputeUnits - c.flat_until) : 0.0;
+  return c;
 }
 inline double tile_round_us(const TileShape& t, int k_tiles, long busy, int row = kCostPlain) {
   const TileCost c = tile_cost(t, row);
@@ -782,7 +796,7 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
   if (streaming_groups > kComputeUnits) {
     streaming_us *= static_cast<double>(rounds) / (static_cast<double>(streaming_groups) / kComputeUnits);
   }
-  if (row == kCostBf16) streaming_us *= 1.06;
+  if (row & kCostBf16) streaming_us *= 1.06;
   return streaming_us < tile_us;
 }
 
