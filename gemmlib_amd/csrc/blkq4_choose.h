@@ -637,7 +637,7 @@ inline double tile_estimate_us(const TileShape& t, int k, int row = kCostPlain) 
 // producer waves): K = 1024 (16 k tiles) 6.5 -> 7.3 us with up to 32 rows, 7.3 -> 9.5 with up to 64; K = 2048 10.0 ->
 // 12.1 and 11.0 -> 15.8; K = 4096 17.5 -> 20.5 and 19.4 -> 27.4; 256 columns with eight waves 28.6 -> 31.7 us at
 // K = 4096.  Whole rounds of 256 workgroups.
-inline double one_row_tile_estimate_us(const TileShape& t, int k) {
+inline double one_row_tile_estimate_us(const TileShape& t, int k, int row = kCostPlain) {
   const long busy = t.tiles < kComputeUnits ? t.tiles : kComputeUnits;
   double step, fixed;
   if (t.wn != 4) {
@@ -649,6 +649,9 @@ inline double one_row_tile_estimate_us(const TileShape& t, int k) {
   } else {
     step = 0.25 + (busy > 128 ? (busy - 128) * 0.00097 : 0.0);
     fixed = 3.3;
+    // the 64 x 128 tile of the general kernel: bf16 and blocks of 16 cost it what they cost there (bf16, M = 48,
+    // N = 14336, K = 4096: 24.4 us unsplit where fp16 takes 19.4, 21.0 against 18.9 in 2 parts)
+    if (row != kCostPlain) step *= tile_cost(t, row).step_idle / tile_cost(t, kCostPlain).step_idle;
   }
   return static_cast<double>(ceil_div(t.tiles, kComputeUnits)) * (fixed + (k / 64) * step);
 }
@@ -658,10 +661,10 @@ inline double one_row_tile_estimate_us(const TileShape& t, int k) {
 // estimated (fp16, blocks of 64) 0 ... -1.3 us at 128 workgroups (N = 4096, K = 4096 ... 14336 in 4 parts), 0.7 at 160,
 // 1.0 ... 1.5 at 172 ... 192 (16 ... 32 k tiles a part), 2.2 ... 2.9 at 216 ... 240, 3.0 and 4.5 at 256 (64 and 112 k
 // tiles a part).
-inline double few_rows_tile_estimate_us(const TileShape& t, int k) {
-  if (t.split_k == 1) return one_row_tile_estimate_us(t, k);
+inline double few_rows_tile_estimate_us(const TileShape& t, int k, int row = kCostPlain) {
+  if (t.split_k == 1) return one_row_tile_estimate_us(t, k, row);
   const long units = static_cast<long>(t.split_tiles) * t.split_k;
-  double us = tile_estimate_us(t, k);
+  double us = tile_estimate_us(t, k, row);
   if (units > 160) us += 1.5 + 0.023 * static_cast<double>(ceil_div(k / 64, t.split_k)) * static_cast<double>(units - 160) / 96.0;
   return us;
 }
@@ -685,14 +688,14 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
   if (column_wise && m <= 64) {
     const int rt = m <= 32 ? 1 : 2;
     const TileShape narrow = shape(rt, 1, 1, 4, 4), wide = shape(rt, 1, 1, 8, 0);
-    // (up to 64 rows the estimates of the tile and of the streaming kernel are those of fp16 for bf16 too: the choice
-    // between them was checked in bf16 on M = 40 and 64 and was within 4 % of the best plan on every shape)
+    // (up to 32 rows the estimates of the tile and of the streaming kernel are those of fp16 with blocks of 64 for
+    // every form)
     TileShape one = one_row_tile_estimate_us(narrow, k) <= one_row_tile_estimate_us(wide, k) ? narrow : wide;
     if (rt == 2) {
       // 33 to 64 rows on a layer that does not fill the chip: the 64 x 128 tile, which is the narrow shape here, has
       // a split form (M = 64, N = 5120, K = 13824: 23.0 us in 4 parts, 30.3 streaming, 55 unsplit; N = 8192, K = 28672:
       // 48.8, 62.9 and 110; N = 16384, K = 8192: 31.8 in 2 parts, 36.0 and 35.2)
-      const double unsplit_us = one_row_tile_estimate_us(one, k);
+      const double unsplit_us = one_row_tile_estimate_us(one, k, row);
       double best_us = unsplit_us;
       TileShape t = narrow;
       for (int split = 2; split <= kMaxSplit; ++split) {
@@ -701,7 +704,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
         t.split_tiles = t.tiles;
         t.workspace_bytes = tile_workspace_bytes(t);
         if (t.workspace_bytes > workspace_capacity || static_cast<size_t>(t.tiles) * sizeof(int) > kCounterBytes) continue;
-        const double us = few_rows_tile_estimate_us(t, k);
+        const double us = few_rows_tile_estimate_us(t, k, row);
         if (us < 0.95 * unsplit_us && us < best_us) {
           one = t;
           best_us = us;
@@ -786,6 +789,9 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
     const double kk = static_cast<double>(k) / 1024.0;
     double streaming_us = 3.2 + static_cast<double>(rounds) * (0.44 + s.nt * (0.69 + 0.37 * kk));
     if (kk > 8.0) streaming_us += static_cast<double>(rounds) * s.nt * 0.0075 * (kk - 8.0) * (kk - 8.0);
+    // (33 to 64 rows, where the tile's estimate knows the form: the streaming kernel takes 1.06 x as long in bf16, 1.13 x
+    // with blocks of 16 and 1.19 x with both as with fp16 and blocks of 64, same plans)
+    if (m > 32) streaming_us *= ((row & kCostBf16) ? 1.06 : 1.0) * ((row & kCostBlocksOf16) ? 1.13 : 1.0);
     return streaming_us < tile_us;
   }
   // more row groups, and blocks along N (from 17 rows on: M = 32, K = 8192, N = 28672 with blocks along N takes 80 us
@@ -812,7 +818,7 @@ inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t wo
   if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k);
   const int row = tile_cost_row(column_wise, bf16, block_size);
   c.t = tile_plan(column_wise, m, n, k, workspace_capacity, row);
-  const double tile_us = (column_wise && m <= 64) ? few_rows_tile_estimate_us(c.t, k) : tile_estimate_us(c.t, k, row);
+  const double tile_us = (column_wise && m <= 64) ? few_rows_tile_estimate_us(c.t, k, m > 32 ? row : kCostPlain) : tile_estimate_us(c.t, k, row);
   c.family = streaming_kernel_takes(column_wise, m, n, k, c.s, tile_us, row) ? kFamilyStreaming : kFamilyTile;
   return c;
 }

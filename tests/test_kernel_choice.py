@@ -122,3 +122,62 @@ def test_wide_layers_give_every_compute_unit_the_same_number_of_tiles(capi):
             workgroups = int(re.search(r"(\d+) workgroups", text).group(1))
             assert 4 <= tiles_per_workgroup <= 7 and workgroups <= 256, (m, n, k, text)
             assert (n // 16 + tiles_per_workgroup - 1) // tiles_per_workgroup <= workgroups, (m, n, k, text)
+
+
+def _plan_as_forced_text(text, m):
+    """the plan text of blkq4_gemm_plan_sm80 -> the plan as blkq4_gemm_with_plan_sm80 takes it (None: not recognised)"""
+    import re
+    t = re.match(r"tile: (\d+) x (\d+), (\d+) \+ (\d+) waves( \(the computing waves split the k tile\))?, (\d+) tiles", text)
+    if t:
+        rows, cols, waves, pw = (int(t.group(i)) for i in (1, 2, 3, 4))
+        parts = re.search(r" in (\d+) parts", text)
+        blocks = re.search(r"blocks of (\d+) x (\d+) tiles per XCD", text)
+        if t.group(5):
+            key = f"tile {rows // 32} {cols // 32} 1 1 {pw} 4 1"
+        else:
+            key = f"tile {rows // 32} {cols // (32 * waves)} 1 {waves} {pw} 1 {parts.group(1) if parts else 1}"
+        if blocks:
+            key += f" {-(-m // rows) // int(blocks.group(1))}"   # row bands = tile rows / tile rows of a block
+        return key
+    s = re.match(r"streaming: (\d+) waves (splitting K|with column tiles of their own), (\d+) column tile\(s\) x (\d+) rows, "
+                 r"(\d+) slices in flight, rows (staged per slice|whole in LDS)", text)
+    if s:
+        waves, nt, rows, depth = int(s.group(1)), int(s.group(3)), int(s.group(4)), int(s.group(5))
+        return (f"streaming {depth} {nt} {rows // 16} {waves} {2 if s.group(6) == 'staged per slice' else 1} "
+                f"{waves if s.group(2) == 'splitting K' else 1}")
+    d = re.match(r"decode( \(blocks along N\))?: (\d+) waves splitting K, (\d+) slices requested by each, "
+                 r"(\d+) column tile\(s\) x (\d+) row\(s\)", text)
+    if d:
+        return f"decode {d.group(5)} {d.group(4)} {d.group(2)} {d.group(3)}"
+    return None
+
+
+def test_chosen_plans_against_times_recorded_on_an_mi355x(capi):
+    """The cost model against measurements, without a GPU: tests/golden/plan_times_mi355x.json holds, for 170 shapes
+    (fp16 and bf16, blocks of 16 / 32 / 64, both blockings, M = 1 ... 2304 on the layers of 7B - 70B models), the measured
+    time of every plan that exists for the shape (tests/golden/make_plan_times.py).  The plan the library chooses has to
+    be within 5 % of the fastest recorded one for nine shapes in ten and never more than a fifth behind: a constant of
+    blkq4_choose.h changed for the worse shows here.  (A plan the measurement did not force is skipped.)"""
+    import json
+    import os
+    rows = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "plan_times_mi355x.json")))
+    judged, behind, worst = 0, [], 1.0
+    for r in rows:
+        text = capi.gemm_plan(r["block_size"], r["column_wise"], r["m"], r["n"], r["k"], r["has_offsets"], r["bf16"])[2]
+        key = _plan_as_forced_text(text, r["m"])
+        assert key is not None, text
+        if key not in r["us"] and " ".join(key.split()[:8]) in r["us"]:
+            key = " ".join(key.split()[:8])   # (the same tiles in the plain order, where the order was not forced)
+        fastest = min(r["us"].values())
+        if key not in r["us"]:
+            if key.startswith("streaming 4 2 1 8 2 8"):
+                continue   # a streaming shape that the measurement does not force
+            ratio = 1.6    # left out of the fixture: more than 1.6 times the fastest
+        else:
+            ratio = r["us"][key] / fastest
+        judged += 1
+        worst = max(worst, ratio)
+        if ratio > 1.05:
+            behind.append((r["bf16"], r["block_size"], r["column_wise"], r["m"], r["n"], r["k"], key, round(ratio, 3)))
+    assert judged >= 160
+    assert len(behind) <= judged // 10 and worst <= 1.2, behind
