@@ -145,13 +145,14 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
   }
   if (!column_wise) {
     // Blocks along N: up to four rows, one column tile per workgroup, eight waves with up to eight slices each
-    // (four waves for short K and for one workgroup per compute unit at most with eight slices each); the scales
+    // (four waves for short K and, with one row, for one workgroup per compute unit at most with eight slices each); the scales
     // and zero-points of a wave's slices, one of each per k, come through LDS.  (M = 1, K = N = 4096: 4.3 against
     // the streaming kernel's 5.3 us.)
     const int slices = k / 128;
     const int tiles = n / 16;
     if (m > 4 || slices > 8 * kDecodeMaxDepth) return false;
-    const int waves = (slices <= 8 || (slices > 28 && slices <= 32 && tiles <= kComputeUnits)) ? 4 : 8;
+    // (two to four rows: eight waves there too, M = 4, K = N = 4096 4.67 against 5.02 us; one row: level, 4.57 and 4.62)
+    const int waves = (slices <= 8 || (m == 1 && slices > 28 && slices <= 32 && tiles <= kComputeUnits)) ? 4 : 8;
     d->row = 1;
     d->rows = m == 1 ? 1 : 4;
     d->nt = 1;

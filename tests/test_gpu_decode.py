@@ -46,6 +46,7 @@ ROW_CASES = [
     (64, False, 1, 4096, 4096), (64, True, 1, 1024, 1024), (32, True, 2, 96, 128), (16, True, 3, 160, 256),
     (32, False, 4, 2080, 384), (64, True, 1, 4160, 2048), (16, False, 1, 704, 3200), (32, True, 4, 1056, 5120),
     (64, False, 2, 1024, 8192), (16, True, 1, 32000, 1152), (64, True, 3, 128, 640), (32, True, 1, 14336, 4096),
+    (64, True, 4, 4096, 4096), (32, False, 2, 2048, 4096),   # two to four rows, 32 slices: eight waves with four each
 ]
 
 
