@@ -138,7 +138,7 @@ inline bool streaming_takes_few_rows(int m, int n, int k) {
 // M = 9 ... 16, K = 4096, N = 14336 9.1 - 9.9 us against the streaming kernel's 10.4 - 10.9, N = 16384 10.1 against 11.1 (at
 // N = 11008 three tiles stay ahead, 8.7 against 9.4); with eight rows a fourth tile gains nothing (N = 14336 8.6 against
 // 8.7 with two, N = 16384 9.6 against 9.0).
-inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) {
+inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d, int block_size = 64) {
   if (m < 1 || m > kDecodeMaxRows || (k % 128) != 0 || (n % 16) != 0 ||
       static_cast<uint64_t>(k) * static_cast<uint64_t>(n) > (uint64_t{1} << 32)) {
     return false;
@@ -171,6 +171,12 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d) 
     if (slices <= 8) waves = 4;
     if (slices > 8 * kDecodeMaxDepth) waves = 16;
     if (slices > 16 * kDecodeMaxDepthSixteenWaves) return false;
+    // K = N = 8192 (512 tiles, 64 slices): sixteen waves with four slices each, two such workgroups per compute unit
+    // and all 512 resident at once, against two rounds of eight waves with eight or one round of two tiles
+    // (M = 1 8.53 against 8.84 us, M = 2 8.88 against 9.99, M = 4 9.38 against 9.78; with 320 ... 448 tiles, N = 5120 ... 7168,
+    // the eight waves stay 0 - 8 % ahead, and so they do with blocks of 16, whose scales are four times as many:
+    // M = 3 11.2 us with two tiles against 12.4)
+    if (waves == 8 && block_size >= 32 && slices > 56 && slices <= 64 && tiles > 448 && tiles <= 2 * kComputeUnits) waves = 16;
   }
   const int depth = (slices + waves - 1) / waves;
   if (depth > ((rows == 16) ? 4 : (rows <= 4 && waves == 16) ? kDecodeMaxDepthSixteenWaves : kDecodeMaxDepth)) return false;
@@ -812,7 +818,7 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
 inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t workspace_capacity, int block_size = 64) {
   Choice c{};
   // few rows, blocks along K, a K that a workgroup can request at once: the decode kernel
-  if (decode_shape(column_wise, m, n, k, &c.d)) {
+  if (decode_shape(column_wise, m, n, k, &c.d, block_size)) {
     c.family = kFamilyDecode;
     return c;
   }

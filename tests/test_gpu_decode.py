@@ -38,6 +38,8 @@ EXACT_CASES = [
     (64, True, 16, 14336, 4096), (32, False, 9, 12320, 4096), (16, True, 12, 13312, 1024), (64, True, 10, 16384, 2176),
     # eight rows, five slices per wave: one workgroup per compute unit, two rounds of them
     (64, True, 8, 13824, 5120), (32, False, 6, 15360, 5120),
+    # up to four rows, 64 slices, 449 to 512 tiles: sixteen waves with four slices each, two workgroups per compute unit
+    (64, True, 2, 8192, 8192), (32, False, 1, 7680, 8192), (32, True, 4, 8192, 7680),
 ]
 
 
