@@ -127,8 +127,9 @@ inline bool streaming_takes_few_rows(int m, int n, int k) {
 // Column tiles per workgroup.  The busiest compute unit works through ceil(workgroups / 256) workgroups of nt
 // tiles each, and every workgroup costs a fraction of a tile's work on top: staging the rows, the instructions
 // before the first request, the sum across the waves.  That fraction, fitted to sweeps over N = 4096 .. 28672 at
-// K = 4096 and 8192: 0.1 for one row, 0.5 for more.  Two tiles with more than four slices per wave take a tenth
-// longer than that (registers: fewer workgroups fit a compute unit).
+// K = 4096 and 8192: 0.1 for one row, 0.5 for more.  Two tiles with more than six slices per wave take a tenth
+// longer than that (registers: fewer workgroups fit a compute unit), with five or six a twenty-fifth (M = 2 ... 4, K = 5120,
+// N = 27648: two tiles 15.5 - 16.1 us, one 16.6 - 17.6).
 //
 // Eight and sixteen rows keep 64 to 128 KiB of rows per workgroup, so one or two workgroups fit a compute unit and a
 // second round of them starts from nothing; once there are more rounds than that the streaming kernel, whose
@@ -188,7 +189,7 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d, 
     if (decode_lds_bytes(false, rows, t, waves, depth) > kMaxLdsBytes) break;
     const int wgs = (tiles + t - 1) / t;
     float cost = static_cast<float>((wgs + kComputeUnits - 1) / kComputeUnits) * (static_cast<float>(t) + per_workgroup);
-    if (rows <= 4 && t == 2 && depth > 4) cost *= 1.1f;
+    if (rows <= 4 && t == 2 && depth > 4) cost *= depth > 6 ? 1.1f : 1.04f;
     if (t == 1 || cost < best) {
       best = cost;
       nt = t;
