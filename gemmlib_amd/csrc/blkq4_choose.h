@@ -107,10 +107,16 @@ inline uint32_t decode_grid(int n, int nt) {
 //     14.9; K = 11008, N = 28672 with zero-points 42.6 -> 37.7, N = 14336 without 19.0 -> 20.6, the one loss found; on
 //     wider layers the decode kernel is ahead again: K = 11008, N = 36864 41.4 against 44.0).
 // At K = 4096 and on wider layers the decode kernel wins.
-inline bool streaming_takes_few_rows(int m, int n, int k) {
+// (The first case later, against the decode kernel's eight waves with eight slices each and one tile per workgroup:
+// with blocks of 32 or 64 two and three rows are 2 - 7 % faster in the decode kernel up to 1792 tiles -- M = 2, K = 8192,
+// N = 22016 21.3 against 23.0 us, N = 28672 26.0 against 27.7 -- four rows level, N = 57344 level to 8 % behind; with blocks
+// of 16 the streaming kernel is 10 - 15 % ahead throughout, N = 24576, M = 4 28.9 against 33.1.)
+inline bool streaming_takes_few_rows(int m, int n, int k, int block_size = 64) {
   const int tiles = n / 16;
   if (m > 4) return false;
-  return (m >= 2 && k >= 8192 && tiles >= 1376 && tiles <= 3584) || (k > 8192 && tiles >= 832 && tiles <= 1792);
+  if (k > 8192 && tiles >= 832 && tiles <= 1792) return true;
+  if (m >= 2 && k >= 8192 && tiles >= 1376 && tiles <= 3584) return block_size < 32 || m == 4 || tiles > 1792;
+  return false;
 }
 
 // The decode kernel's shape for m rows, or false when it has none or the streaming kernel is expected to be
@@ -129,7 +135,8 @@ inline bool streaming_takes_few_rows(int m, int n, int k) {
 // before the first request, the sum across the waves.  That fraction, fitted to sweeps over N = 4096 .. 28672 at
 // K = 4096 and 8192: 0.1 for one row, 0.5 for more.  Two tiles with more than six slices per wave take a tenth
 // longer than that (registers: fewer workgroups fit a compute unit), with five or six a twenty-fifth (M = 2 ... 4, K = 5120,
-// N = 27648: two tiles 15.5 - 16.1 us, one 16.6 - 17.6).
+// N = 27648: two tiles 15.5 - 16.1 us, one 16.6 - 17.6), and two fifths longer when they need more than one round (K = 8192,
+// M = 2: N = 14336 17.8 us against 15.2 with one tile, N = 28672 34.5 against 26.0).
 //
 // Eight and sixteen rows keep 64 to 128 KiB of rows per workgroup, so one or two workgroups fit a compute unit and a
 // second round of them starts from nothing; once there are more rounds than that the streaming kernel, whose
@@ -165,7 +172,7 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d, 
   }
   const int slices = k / 128;
   const int tiles = n / 16;
-  if (streaming_takes_few_rows(m, n, k)) return false;
+  if (streaming_takes_few_rows(m, n, k, block_size)) return false;
   const int rows = m == 1 ? 1 : m <= 4 ? 4 : m <= 8 ? 8 : 16;
   int waves = 8;
   if (rows <= 4) {
@@ -189,7 +196,7 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d, 
     if (decode_lds_bytes(false, rows, t, waves, depth) > kMaxLdsBytes) break;
     const int wgs = (tiles + t - 1) / t;
     float cost = static_cast<float>((wgs + kComputeUnits - 1) / kComputeUnits) * (static_cast<float>(t) + per_workgroup);
-    if (rows <= 4 && t == 2 && depth > 4) cost *= depth > 6 ? 1.1f : 1.04f;
+    if (rows <= 4 && t == 2 && depth > 4) cost *= depth <= 6 ? 1.04f : wgs <= kComputeUnits ? 1.1f : 1.4f;
     if (t == 1 || cost < best) {
       best = cost;
       nt = t;
@@ -319,7 +326,7 @@ inline void streaming_geometry(StreamingShape* s, bool row, int n, int k) {
   s->refill = (cg_stride < col_groups || s->split == 1) ? 1 : 0;
 }
 
-inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
+inline StreamingShape streaming_shape(bool row, int m, int n, int k, int block_size = 64) {
   StreamingShape s{};
   auto set = [&](int depth, int nt, int mt, int waves, int am, int split) {
     s.depth = depth; s.nt = nt; s.mt = mt; s.waves = waves; s.am = am; s.split = split;
@@ -391,7 +398,7 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k) {
       return done();
     }
   }
-  if (!row && (!rows_fit || m > 4 || streaming_takes_few_rows(m, n, k)) && k >= 1024) {
+  if (!row && (!rows_fit || m > 4 || streaming_takes_few_rows(m, n, k, block_size)) && k >= 1024) {
     // Wide N and more than four rows, or K too long for the rows to stay in LDS: the rows are staged per
     // slice, a workgroup takes four column tiles (the rows are fetched again for every column group) and a
     // wave keeps two slices in flight, so that the slots are small enough for several workgroups per compute
@@ -823,7 +830,7 @@ inline Choice choose(bool column_wise, bool bf16, int m, int n, int k, size_t wo
     c.family = kFamilyDecode;
     return c;
   }
-  if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k);
+  if (m <= kStreamingMaxRows) c.s = streaming_shape(!column_wise, m, n, k, block_size);
   const int row = tile_cost_row(column_wise, bf16, block_size);
   c.t = tile_plan(column_wise, m, n, k, workspace_capacity, row);
   const double tile_us = (column_wise && m <= 64) ? few_rows_tile_estimate_us(c.t, k, m > 32 ? row : kCostPlain) : tile_estimate_us(c.t, k, row);
