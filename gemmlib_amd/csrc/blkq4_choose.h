@@ -135,8 +135,9 @@ inline bool streaming_takes_few_rows(int m, int n, int k, int block_size = 64) {
 // before the first request, the sum across the waves.  That fraction, fitted to sweeps over N = 4096 .. 28672 at
 // K = 4096 and 8192: 0.1 for one row, 0.5 for more.  Two tiles with more than six slices per wave take a tenth
 // longer than that (registers: fewer workgroups fit a compute unit), with five or six a twenty-fifth (M = 2 ... 4, K = 5120,
-// N = 27648: two tiles 15.5 - 16.1 us, one 16.6 - 17.6), and two fifths longer when they need more than one round (K = 8192,
-// M = 2: N = 14336 17.8 us against 15.2 with one tile, N = 28672 34.5 against 26.0).
+// N = 27648: two tiles 15.5 - 16.1 us, one 16.6 - 17.6), and with eight two fifths longer when they need more than one
+// round (K = 8192, M = 2: N = 14336 17.8 us against 15.2 with one tile, N = 28672 34.5 against 26.0; with seven slices,
+// K = 7168, N = 32768, M = 3, two tiles take 24.2 us and one 27.6).
 //
 // Eight and sixteen rows keep 64 to 128 KiB of rows per workgroup, so one or two workgroups fit a compute unit and a
 // second round of them starts from nothing; once there are more rounds than that the streaming kernel, whose
@@ -196,7 +197,7 @@ inline bool decode_shape(bool column_wise, int m, int n, int k, DecodeShape* d, 
     if (decode_lds_bytes(false, rows, t, waves, depth) > kMaxLdsBytes) break;
     const int wgs = (tiles + t - 1) / t;
     float cost = static_cast<float>((wgs + kComputeUnits - 1) / kComputeUnits) * (static_cast<float>(t) + per_workgroup);
-    if (rows <= 4 && t == 2 && depth > 4) cost *= depth <= 6 ? 1.04f : wgs <= kComputeUnits ? 1.1f : 1.4f;
+    if (rows <= 4 && t == 2 && depth > 4) cost *= depth <= 6 ? 1.04f : (depth < 8 || wgs <= kComputeUnits) ? 1.1f : 1.4f;
     if (t == 1 || cost < best) {
       best = cost;
       nt = t;
