@@ -359,7 +359,9 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k, int block_s
         }
       }
     }
-    const bool rows_fit = static_cast<size_t>(k) * 2 * 32 <= kMaxLdsBytes;
+    // the rows whole in LDS only while they are a small part of it: at K = 2048 (128 KB) staging them slice by slice is
+    // a tenth faster (M = 80 ... 128, N = 4096: 7.4 - 7.6 against 8.2 - 8.3 us), at K = 1024 they are level
+    const bool rows_fit = static_cast<size_t>(k) * 2 * 32 <= kMaxLdsBytes && k <= 1536;
     set(2, nt, 2, 8, rows_fit ? kRowsWholeInLds : kRowsPerSlotInLds, 8);
     streaming_geometry(&s, row, n, k);
     return s;
@@ -793,7 +795,10 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
   const long rounds = s.cg_stride >= col_groups
                           ? streaming_rounds(s.row_groups, static_cast<int>(col_groups), streaming_neighbours(s.nt, s.waves, s.split))
                           : ceil_div(streaming_groups, kComputeUnits);
-  if (column_wise && m <= 64) {
+  if (column_wise && (m <= 64 || k < 4096)) {
+    // (More row groups with a short K too: the product further down has no fixed part and said 5.6 us for M = 256,
+    // K = 1024, N = 4096, which takes 11.3 -- and the 128 x 32 tiles whose waves split the k tile 6.7; this line says 12.1.
+    // Of 63 shapes with M = 80 ... 384, K = 1024 ... 3072 sixteen went to the streaming kernel and lost 8 - 70 % by it.)
     // One or two row groups of 32, blocks along K: rounds of 256 workgroups, a workgroup's time growing with its
     // column tiles and K.  Least squares over 142 measurements (M = 24 ... 64, K = 1024 ... 4096, N = 2048 ... 32768;
     // within 15 % of all but a few, and of M = 128, K = N = 4096 and M = 40 ... 64, K = 8192, N = 16384 ... 18432, which
