@@ -361,7 +361,8 @@ inline StreamingShape streaming_shape(bool row, int m, int n, int k, int block_s
     }
     // the rows whole in LDS only while they are a small part of it: at K = 2048 (128 KB) staging them slice by slice is
     // a tenth faster (M = 80 ... 128, N = 4096: 7.4 - 7.6 against 8.2 - 8.3 us), at K = 1024 they are level
-    const bool rows_fit = static_cast<size_t>(k) * 2 * 32 <= kMaxLdsBytes && k <= 1536;
+    // (blocks along K; with blocks along N whole rows stay ahead, M = 24 ... 96, K = 2048: 8.1 - 11.6 against 9.8 - 15.7 us)
+    const bool rows_fit = static_cast<size_t>(k) * 2 * 32 <= kMaxLdsBytes && (row || k <= 1536);
     set(2, nt, 2, 8, rows_fit ? kRowsWholeInLds : kRowsPerSlotInLds, 8);
     streaming_geometry(&s, row, n, k);
     return s;
@@ -814,6 +815,17 @@ inline bool streaming_kernel_takes(bool column_wise, int m, int n, int k, const 
     // with blocks of 16 and 1.19 x with both as with fp16 and blocks of 64, same plans)
     if (m > 32) streaming_us *= ((row & kCostBf16) ? 1.06 : 1.0) * ((row & kCostBlocksOf16) ? 1.13 : 1.0);
     return streaming_us < tile_us;
+  }
+  if (!column_wise && k < 4096) {
+    // Blocks along N with a short K: one column tile per workgroup, so row groups x N / 16 workgroups, and the time grows
+    // with their number per compute unit: measured 2.5 us + (row groups x N / 4096) x 2.5 (K = 1024) or 2.8 (K = 2048)
+    // with the rows whole in LDS (M = 24 ... 96, N = 4096 and 8192: 5.0 ... 17.4 and 5.3 ... 18.4 us), 6 at K = 4096 where they
+    // are staged per slice.  (The product below said 5.6 us for M = 48, N = 8192, K = 1024, which takes 12.6; tiles 8.2.)
+    // The tiles' estimate is the less certain one at this size: the streaming kernel keeps what it wins by less than 15 %.
+    const double x = static_cast<double>(row_groups) * (static_cast<double>(n) / 4096.0);
+    const double kk = static_cast<double>(k) / 1024.0;
+    const double streaming_us = 2.5 + x * (k <= 2560 ? 2.2 + 0.3 * kk : 1.5 * kk);
+    return streaming_us < 1.15 * tile_us;
   }
   // more row groups, and blocks along N (from 17 rows on: M = 32, K = 8192, N = 28672 with blocks along N takes 80 us
   // streaming and 50 in 64 x 128 tiles), where the streaming kernel converts with 23 instead of 13 instructions per 8
