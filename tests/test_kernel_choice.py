@@ -153,8 +153,8 @@ def _plan_as_forced_text(text, m):
 
 
 def test_chosen_plans_against_times_recorded_on_an_mi355x(capi):
-    """The cost model against measurements, without a GPU: tests/golden/plan_times_mi355x.json holds, for 170 shapes
-    (fp16 and bf16, blocks of 16 / 32 / 64, both blockings, M = 1 ... 2304 on the layers of 7B - 70B models), the measured
+    """The cost model against measurements, without a GPU: tests/golden/plan_times_mi355x.json holds, for 311 shapes
+    (fp16 and bf16, blocks of 16 / 32 / 64, both blockings, M = 1 ... 2304 on the layers of 7B - 70B models, K from 1024), the measured
     time of every plan that exists for the shape (tests/golden/make_plan_times.py).  The plan the library chooses has to
     be within 5 % of the fastest recorded one for nine shapes in ten and never more than a fifth behind: a constant of
     blkq4_choose.h changed for the worse shows here.  (A plan the measurement did not force is skipped.)"""
@@ -179,5 +179,5 @@ def test_chosen_plans_against_times_recorded_on_an_mi355x(capi):
         worst = max(worst, ratio)
         if ratio > 1.05:
             behind.append((r["bf16"], r["block_size"], r["column_wise"], r["m"], r["n"], r["k"], key, round(ratio, 3)))
-    assert judged >= 160
+    assert judged >= 300
     assert len(behind) <= judged // 10 and worst <= 1.2, behind
