@@ -719,6 +719,7 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
       TileShape t = narrow;
       for (int split = 2; split <= kMaxSplit; ++split) {
         if (t.tiles * split > kComputeUnits || kt / split < kMinKTilesPerPart) break;
+        if (split == 4 && t.tiles * 4 > 224 && kt < 128) continue;  // (as for more rows, below)
         t.split_k = split;
         t.split_tiles = t.tiles;
         t.workspace_bytes = tile_workspace_bytes(t);
@@ -760,6 +761,11 @@ inline TileShape tile_plan(bool column_wise, int m, int n, int k, size_t workspa
     if (rem == 0) continue;
     for (int split = 2; split <= kMaxSplit; ++split) {
       if (rem * split > kComputeUnits || kt / split < kMinKTilesPerPart) break;
+      // A fourth part that fills the chip pays only with a long K: of 86 problems measured with 64 tiles in 4 parts, three
+      // parts are faster for most below K = 8192 (median 6 %), four by 3 - 13 % at K = 11008; and with every compute unit
+      // busy the last workgroups' invalidates hit the others' operands (M = 256, K = N = 4096, blocks along N, 128 x 128
+      // tiles: 25 - 27 us in 4 parts on one box of the pool, 20.6 on the others, 20.2 in 3 parts on all).
+      if (split == 4 && rem * 4 > 224 && kt < 128) continue;
       t.split_k = split;
       t.split_tiles = rem;
       t.workspace_bytes = tile_workspace_bytes(t);
